@@ -1,0 +1,451 @@
+// Flash attention forward for gfx950, head dim 128, bf16 operands, fp32 online softmax.
+//
+// Work split: one workgroup = 4 waves = 256 consecutive query rows of one (batch, head);
+// every wave owns 64 queries (two 32-wide MFMA column tiles) and walks all keys in blocks of 64.
+//
+// MFMA formulation (v_mfma_f32_32x32x16_bf16, D[i][j] += sum_k A[i][k] * B[k][j]; lane (g,i)
+// feeds A[i][8g..8g+7], lane (g,j) feeds B[8g..8g+7][j]; result lane (g,j) register r holds
+// row 8*(r/4) + 4g + (r%4), column j):
+//   S^T = K * Q^T      A = K tile (from LDS), B = Q^T (registers, loaded once)
+//   O^T += V^T * P^T   A = V^T tile (from LDS), B = P^T (registers, straight from S^T)
+// With the transposed formulation a lane only ever holds data of ONE query (column j), so the
+// softmax row statistics are lane-local apart from one exchange between the two half-waves,
+// and the S^T accumulators turn into the B operand of the second product without any shuffle:
+// registers 8c..8c+7 of an S^T tile are keys {4g..4g+3, 8+4g..8+4g+3} of 16-key chunk c, and the
+// V^T tile in LDS stores its key axis in exactly that slot order.
+//
+// LDS per stage: K tile [64 keys][128 d] (256-byte rows, 16-byte chunk c of row r stored at
+// c ^ (r & 15)) and V^T tile [128 d][64 key slots] (128-byte rows, chunk c of row r stored at
+// c ^ ((r/2) & 7)); both swizzles make 16 consecutive rows at one logical chunk conflict-free.
+#include "common.h"
+
+namespace dsx {
+
+constexpr int QB = 256;   // queries per workgroup
+constexpr int KB = 64;    // keys per block
+constexpr int HD = 128;   // head dim
+constexpr int kKTileBytes = KB * HD * 2;          // 16 KiB
+constexpr int kAttnStageBytes = 2 * kKTileBytes;  // K + V^T
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ int k_lds_off(int key, int chunk) {
+  return key * 256 + ((chunk ^ (key & 15)) << 4);
+}
+__device__ __forceinline__ int vt_lds_off(int d, int chunk) {
+  return d * 128 + ((chunk ^ ((d >> 1) & 7)) << 4);
+}
+
+__device__ __forceinline__ float halfwave_allmax(float v) {
+  // max over the pair of lanes (l, l^32)
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halfwave_allsum(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// RMSNorm + RoPE on 8 consecutive head-dim elements (pairs 4c..4c+3 of the row), given the
+// reciprocal rms of the whole row.  Rounding points follow the bf16 torch sequence:
+// bf16(x * rrms) -> bf16(. * w) -> fp32 rotate -> bf16.
+__device__ __forceinline__ u32x4 norm_rope_chunk(u32x4 raw, bool has_norm, float rrms,
+                                                 const uint16_t* __restrict__ w8,
+                                                 const float* __restrict__ cs8) {
+  float v[8];
+  v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x); v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);
+  v[4] = bf16_lo(raw.z); v[5] = bf16_hi(raw.z); v[6] = bf16_lo(raw.w); v[7] = bf16_hi(raw.w);
+  if (has_norm) {
+    u32x4 wv = *reinterpret_cast<const u32x4*>(w8);
+    float wf[8] = {bf16_lo(wv.x), bf16_hi(wv.x), bf16_lo(wv.y), bf16_hi(wv.y),
+                   bf16_lo(wv.z), bf16_hi(wv.z), bf16_lo(wv.w), bf16_hi(wv.w)};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = round_bf16(round_bf16(v[i] * rrms) * wf[i]);
+  }
+  if (cs8) {
+    f32x4 t0 = *reinterpret_cast<const f32x4*>(cs8);
+    f32x4 t1 = *reinterpret_cast<const f32x4*>(cs8 + 4);
+    float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float c = cs[2 * i], s = cs[2 * i + 1];
+      float x0 = v[2 * i], x1 = v[2 * i + 1];
+      // same expression order as freqs[...,0]*x0 + freqs[...,1]*x1 with rows (c,-s) and (s,c)
+      // (separately rounded products and sum, as separate torch ops produce them)
+      v[2 * i] = __fadd_rn(__fmul_rn(c, x0), __fmul_rn(-s, x1));
+      v[2 * i + 1] = __fadd_rn(__fmul_rn(s, x0), __fmul_rn(c, x1));
+    }
+  }
+  u32x4 o;
+  o.x = pack_bf16x2(v[0], v[1]);
+  o.y = pack_bf16x2(v[2], v[3]);
+  o.z = pack_bf16x2(v[4], v[5]);
+  o.w = pack_bf16x2(v[6], v[7]);
+  return o;
+}
+
+__device__ __forceinline__ float sumsq_chunk(u32x4 raw) {
+  float s = 0.f;
+  float a;
+  a = bf16_lo(raw.x); s += a * a; a = bf16_hi(raw.x); s += a * a;
+  a = bf16_lo(raw.y); s += a * a; a = bf16_hi(raw.y); s += a * a;
+  a = bf16_lo(raw.z); s += a * a; a = bf16_hi(raw.z); s += a * a;
+  a = bf16_lo(raw.w); s += a * a; a = bf16_hi(raw.w); s += a * a;
+  return s;
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int g = lane >> 5, li = lane & 31;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int64_t Sq = p.sq[0] + p.sq[1];
+  const int64_t Skv = p.skv[0] + p.skv[1];
+  const int64_t q0 = (int64_t)blockIdx.x * QB + wave * 64;
+
+  const uint16_t* qbase[2] = {(const uint16_t*)p.q[0], (const uint16_t*)p.q[1]};
+  const uint16_t* kbase[2] = {(const uint16_t*)p.k[0], (const uint16_t*)p.k[1]};
+  const uint16_t* vbase[2] = {(const uint16_t*)p.v[0], (const uint16_t*)p.v[1]};
+  const int64_t q_bh = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+  const int64_t k_bh = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+  const int64_t v_bh = (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+  const float* rope = FUSED && p.rope ? p.rope + (int64_t)b * p.rope_sb : nullptr;
+
+  // ---------------- Q fragments (B operand of S^T = K Q^T), loaded once ----------------
+  bf16x8 qf[2][8];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    int64_t row = q0 + qt * 32 + li;
+    if (row >= Sq) row = Sq - 1;
+    const int seg = row >= p.sq[0] ? 1 : 0;
+    const uint16_t* src = qbase[seg] + q_bh + (row - (seg ? p.sq[0] : 0)) * p.q_ss;
+    u32x4 raw[8];
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) raw[kc] = *reinterpret_cast<const u32x4*>(src + kc * 16 + g * 8);
+    if (FUSED) {
+      const uint16_t* nw = (const uint16_t*)p.q_norm_w[seg];
+      float rrms = 1.f;
+      if (nw) {
+        float ss = 0.f;
+#pragma unroll
+        for (int kc = 0; kc < 8; ++kc) ss += sumsq_chunk(raw[kc]);
+        ss = halfwave_allsum(ss);
+        rrms = rsqrtf(ss * (1.0f / HD) + p.norm_eps);
+      }
+#pragma unroll
+      for (int kc = 0; kc < 8; ++kc)
+        raw[kc] = norm_rope_chunk(raw[kc], nw != nullptr, rrms, nw ? nw + kc * 16 + g * 8 : nullptr,
+                                  rope ? rope + row * HD + kc * 16 + g * 8 : nullptr);
+    }
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) qf[qt][kc] = __builtin_bit_cast(bf16x8, raw[kc]);
+  }
+
+  // ---------------- K / V staging maps ----------------
+  // K: chunk id = tid + 256*i -> key = id/16, chunk = id%16 (16 lanes read one 256-byte row)
+  const int ks_c = tid & 15;
+  const int ks_r = tid >> 4;  // +16*i
+  // V: thread owns 4 keys x 8 d: dgroup = tid%16, keygroup = tid/16
+  const int vs_dg = tid & 15;
+  const int vs_kg = tid >> 4;
+  // destination of the transposed 8-byte pieces: 16-key chunk ch, kappa0 = 4*(kg%4) = 8a + 4gg
+  const int vs_ch = vs_kg >> 2;
+  const int vs_a = (vs_kg >> 1) & 1;
+  const int vs_gg = vs_kg & 1;
+  const int vs_chunk = vs_ch * 2 + vs_gg;
+
+  u32x4 sk[4], sv[4];
+  auto load_kv = [&](int kb) {
+    const int64_t key0 = (int64_t)kb * KB;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int64_t key = key0 + ks_r + 16 * i;
+      if (key >= Skv) key = Skv - 1;
+      const int seg = key >= p.skv[0] ? 1 : 0;
+      const int64_t lrow = key - (seg ? p.skv[0] : 0);
+      u32x4 raw = *reinterpret_cast<const u32x4*>(kbase[seg] + k_bh + lrow * p.k_ss + ks_c * 8);
+      if (FUSED) {
+        const uint16_t* nw = (const uint16_t*)p.k_norm_w[seg];
+        float rrms = 1.f;
+        if (nw) {
+          float ss = sumsq_chunk(raw);
+          // the 16 lanes tid%16 of one key hold the whole 128-wide row
+          ss += __shfl_xor(ss, 1, 64);
+          ss += __shfl_xor(ss, 2, 64);
+          ss += __shfl_xor(ss, 4, 64);
+          ss += __shfl_xor(ss, 8, 64);
+          rrms = rsqrtf(ss * (1.0f / HD) + p.norm_eps);
+        }
+        raw = norm_rope_chunk(raw, nw != nullptr, rrms, nw ? nw + ks_c * 8 : nullptr,
+                              rope ? rope + key * HD + ks_c * 8 : nullptr);
+      }
+      sk[i] = raw;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int64_t key = key0 + vs_kg * 4 + i;
+      if (key >= Skv) key = Skv - 1;
+      const int seg = key >= p.skv[0] ? 1 : 0;
+      const int64_t lrow = key - (seg ? p.skv[0] : 0);
+      sv[i] = *reinterpret_cast<const u32x4*>(vbase[seg] + v_bh + lrow * p.v_ss + vs_dg * 8);
+    }
+  };
+  auto store_kv = [&](int buf) {
+    uint8_t* sK = smem + buf * kAttnStageBytes;
+    uint8_t* sV = sK + kKTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<u32x4*>(sK + k_lds_off(ks_r + 16 * i, ks_c)) = sk[i];
+      // 4 keys x 8 d  ->  8 d-rows x 4 keys
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t w0 = sv[0][j], w1 = sv[1][j], w2 = sv[2][j], w3 = sv[3][j];
+      u32x2 even, odd;
+      even.x = (w0 & 0xffffu) | (w1 << 16);
+      even.y = (w2 & 0xffffu) | (w3 << 16);
+      odd.x = (w0 >> 16) | (w1 & 0xffff0000u);
+      odd.y = (w2 >> 16) | (w3 & 0xffff0000u);
+      const int d = vs_dg * 8 + 2 * j;
+      *reinterpret_cast<u32x2*>(sV + vt_lds_off(d, vs_chunk) + vs_a * 8) = even;
+      *reinterpret_cast<u32x2*>(sV + vt_lds_off(d + 1, vs_chunk) + vs_a * 8) = odd;
+    }
+  };
+
+  f32x16 oacc[4][2];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[dt][qt][r] = 0.f;
+  float m_run[2] = {-INFINITY, -INFINITY};
+  float l_run[2] = {0.f, 0.f};
+  const float c = p.softmax_scale * kLog2e;
+
+  const int nkb = (int)((Skv + KB - 1) / KB);
+  load_kv(0);
+  store_kv(0);
+  __syncthreads();
+
+  for (int kb = 0; kb < nkb; ++kb) {
+    const int buf = kb & 1;
+    if (kb + 1 < nkb) load_kv(kb + 1);
+    const uint8_t* sK = smem + buf * kAttnStageBytes;
+    const uint8_t* sV = sK + kKTileBytes;
+
+    // ---- S^T = K Q^T
+    f32x16 s[2][2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[kt][qt][r] = 0.f;
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + k_lds_off(kt * 32 + li, 2 * kc + g));
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+          s[kt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qt][kc], s[kt][qt], 0, 0, 0);
+      }
+    }
+    // ---- mask the ragged tail of the key axis
+    if ((int64_t)(kb + 1) * KB > Skv) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t key = (int64_t)kb * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (key >= Skv) {
+            s[kt][0][r] = -INFINITY;
+            s[kt][1][r] = -INFINITY;
+          }
+        }
+    }
+    // ---- online softmax, one query per lane pair (l, l^32)
+    bf16x8 pf[2][2][2];  // [kt][chunk][qt]
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      float mx = s[0][qt][0];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][qt][r]);
+      mx = halfwave_allmax(mx);
+      const float m_new = fmaxf(m_run[qt], mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * c);
+      const float mc = m_new * c;
+      m_run[qt] = m_new;
+      float lsum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        float pv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          pv[r] = __builtin_amdgcn_exp2f(s[kt][qt][r] * c - mc);
+          lsum += pv[r];
+        }
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+          u32x4 w;
+          w.x = pack_bf16x2(pv[8 * ch + 0], pv[8 * ch + 1]);
+          w.y = pack_bf16x2(pv[8 * ch + 2], pv[8 * ch + 3]);
+          w.z = pack_bf16x2(pv[8 * ch + 4], pv[8 * ch + 5]);
+          w.w = pack_bf16x2(pv[8 * ch + 6], pv[8 * ch + 7]);
+          pf[kt][ch][qt] = __builtin_bit_cast(bf16x8, w);
+        }
+      }
+      l_run[qt] = l_run[qt] * alpha + lsum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[dt][qt][r] *= alpha;
+      }
+    }
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int ch = 0; ch < 2; ++ch)
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+          bf16x8 vf =
+              *reinterpret_cast<const bf16x8*>(sV + vt_lds_off(dt * 32 + li, (kt * 2 + ch) * 2 + g));
+#pragma unroll
+          for (int qt = 0; qt < 2; ++qt)
+            oacc[dt][qt] =
+                __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][ch][qt], oacc[dt][qt], 0, 0, 0);
+        }
+
+    if (kb + 1 < nkb) store_kv(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---------------- normalise and store.  lane (g, j): query j, d = dt*32 + 8*(r/4) + 4g + r%4
+  uint16_t* obase[2] = {(uint16_t*)p.o[0], (uint16_t*)p.o[1]};
+  const int64_t o_bh = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const float l = halfwave_allsum(l_run[qt]);
+    const float inv = 1.0f / l;
+    const int64_t row = q0 + qt * 32 + li;
+    if (row < Sq) {
+      const int seg = row >= p.sq[0] ? 1 : 0;
+      uint16_t* dst = obase[seg] + o_bh + (row - (seg ? p.sq[0] : 0)) * p.o_ss;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          u32x2 w;
+          w.x = pack_bf16x2(oacc[dt][qt][4 * rq + 0] * inv, oacc[dt][qt][4 * rq + 1] * inv);
+          w.y = pack_bf16x2(oacc[dt][qt][4 * rq + 2] * inv, oacc[dt][qt][4 * rq + 3] * inv);
+          *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w;
+        }
+    }
+  }
+}
+
+// Standalone RMSNorm + RoPE: one wave per (b,h,s) row... 16 lanes per row, 4 rows per wave.
+__global__ __launch_bounds__(256) void rmsnorm_rope_kernel(
+    const uint16_t* __restrict__ x, int64_t x_sb, int64_t x_sh, int64_t x_ss,
+    const uint16_t* __restrict__ norm_w, float eps, const float* __restrict__ rope, int64_t rope_sb,
+    int64_t rope_pos0, uint16_t* __restrict__ out, int64_t o_sb, int64_t o_sh, int64_t o_ss,
+    int heads, int64_t seq) {
+  const int c = threadIdx.x & 15;
+  const int64_t s = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int h = blockIdx.y, b = blockIdx.z;
+  const bool ok = s < seq;
+  const int64_t sr = ok ? s : seq - 1;
+  u32x4 raw = *reinterpret_cast<const u32x4*>(x + b * x_sb + h * x_sh + sr * x_ss + c * 8);
+  float rrms = 1.f;
+  if (norm_w) {
+    float ss = sumsq_chunk(raw);
+    ss += __shfl_xor(ss, 1, 64);
+    ss += __shfl_xor(ss, 2, 64);
+    ss += __shfl_xor(ss, 4, 64);
+    ss += __shfl_xor(ss, 8, 64);
+    rrms = rsqrtf(ss * (1.0f / HD) + eps);
+  }
+  u32x4 o = norm_rope_chunk(raw, norm_w != nullptr, rrms, norm_w ? norm_w + c * 8 : nullptr,
+                            rope ? rope + b * rope_sb + (rope_pos0 + sr) * HD + c * 8 : nullptr);
+  if (ok) *reinterpret_cast<u32x4*>(out + b * o_sb + h * o_sh + s * o_ss + c * 8) = o;
+}
+
+}  // namespace dsx
+
+static int check_seg(const void* const* ptr, const int64_t* len) {
+  for (int g = 0; g < 2; ++g) {
+    if (len[g] < 0) return DSX_EBADSHAPE;
+    if (len[g] > 0 && !ptr[g]) return DSX_ENULL;
+    if (((uintptr_t)ptr[g]) & 15) return DSX_EALIGN;
+  }
+  return DSX_OK;
+}
+
+extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
+  using namespace dsx;
+  if (!p) return DSX_ENULL;
+  if (p->head_dim != HD || p->batch <= 0 || p->heads <= 0) return DSX_EBADSHAPE;
+  if (p->batch > 65535 || p->heads > 65535) return DSX_EBADSHAPE;
+  int rc;
+  if ((rc = check_seg(p->q, p->sq)) || (rc = check_seg(p->k, p->skv)) ||
+      (rc = check_seg(p->v, p->skv)) || (rc = check_seg((const void* const*)p->o, p->sq)))
+    return rc;
+  const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
+  if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 31) || Skv > (1ll << 31)) return DSX_EBADSHAPE;
+  const int64_t strides[12] = {p->q_sb, p->q_sh, p->q_ss, p->k_sb, p->k_sh, p->k_ss,
+                               p->v_sb, p->v_sh, p->v_ss, p->o_sb, p->o_sh, p->o_ss};
+  for (int i = 0; i < 12; ++i)
+    if (strides[i] & 7) return DSX_EALIGN;  // every row start must stay 16-byte aligned
+  if (p->q_ss < HD && Sq > 1) return DSX_EBADSHAPE;
+  if (p->o_ss < HD && Sq > 1) return DSX_EBADSHAPE;
+  const bool fused = p->rope || p->q_norm_w[0] || p->q_norm_w[1] || p->k_norm_w[0] || p->k_norm_w[1];
+  if (p->rope && (((uintptr_t)p->rope & 15) || (p->rope_sb & 3))) return DSX_EALIGN;
+  if (p->rope && Sq != Skv) return DSX_EBADSHAPE;  // fused RoPE is defined for self/joint attention
+  for (int g = 0; g < 2; ++g)
+    if (((uintptr_t)p->q_norm_w[g] & 15) || ((uintptr_t)p->k_norm_w[g] & 15)) return DSX_EALIGN;
+
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)attn_fwd_kernel<false>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            2 * kAttnStageBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)attn_fwd_kernel<true>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            2 * kAttnStageBytes) != hipSuccess)
+      return DSX_ELAUNCH;
+    attr_set = true;
+  }
+  dim3 grid((unsigned)((Sq + QB - 1) / QB), (unsigned)p->heads, (unsigned)p->batch), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (fused)
+    attn_fwd_kernel<true><<<grid, block, 2 * kAttnStageBytes, st>>>(*p);
+  else
+    attn_fwd_kernel<false><<<grid, block, 2 * kAttnStageBytes, st>>>(*p);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss,
+                                const void* norm_w, float eps, const float* rope, int64_t rope_sb,
+                                int64_t rope_pos0, void* out, int64_t o_sb, int64_t o_sh,
+                                int64_t o_ss, int32_t batch, int32_t heads, int64_t seq,
+                                void* stream) {
+  using namespace dsx;
+  if (!x || !out) return DSX_ENULL;
+  if (batch <= 0 || heads <= 0 || seq < 0 || batch > 65535 || heads > 65535) return DSX_EBADSHAPE;
+  if ((x_sb | x_sh | x_ss | o_sb | o_sh | o_ss) & 7) return DSX_EALIGN;
+  if (((uintptr_t)x & 15) || ((uintptr_t)out & 15) || ((uintptr_t)norm_w & 15) ||
+      ((uintptr_t)rope & 15) || (rope_sb & 3))
+    return DSX_EALIGN;
+  if (seq == 0) return DSX_OK;
+  dim3 grid((unsigned)((seq + 15) / 16), (unsigned)heads, (unsigned)batch), block(256);
+  rmsnorm_rope_kernel<<<grid, block, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)x, x_sb, x_sh, x_ss, (const uint16_t*)norm_w, eps, rope, rope_sb, rope_pos0,
+      (uint16_t*)out, o_sb, o_sh, o_ss, heads, seq);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}

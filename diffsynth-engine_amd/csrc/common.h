@@ -1,0 +1,104 @@
+// Shared device helpers for the gfx950 kernels: vector types, bf16/e4m3 conversion with
+// explicit rounding points, wave64 reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dsx.h"
+
+namespace dsx {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// fp32 -> bf16 bits, round-to-nearest-even, NaN kept quiet (same result as torch's cast).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// Round an fp32 value to the nearest bf16 and return it widened again (an in-register
+// "rounding point" reproducing an intermediate bf16 tensor of the torch op sequence).
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+// Two fp32 -> packed bf16 pair with the hardware converter (v_cvt_pk_bf16_f32, RNE).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Unpack the two bf16 halves of a 32-bit word.
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// fp32 -> OCP e4m3fn, round-to-nearest-even, subnormals kept (step 2^-9), no saturation:
+// |v| >= 480 (everything that does not round to <= 448) and NaN give 0x7f | sign, like
+// torch.Tensor.to(torch.float8_e4m3fn).
+__device__ __forceinline__ uint32_t f32_to_e4m3_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t sign = (u >> 24) & 0x80u;
+  u &= 0x7fffffffu;
+  uint32_t r;
+  if (u >= 0x43f00000u) {            // |f| >= 480 (incl. inf/NaN): not representable
+    r = 0x7fu;
+  } else if (u < 0x3c800000u) {      // |f| < 2^-6: subnormal range, quantum 2^-9
+    // adding 2^14 aligns the quantum 2^-9 with the fp32 ulp at 2^14 (2^-9); the FPU rounds RNE
+    float t = __uint_as_float(u) + 16384.0f;
+    r = __float_as_uint(t) - 0x46800000u;
+  } else {
+    uint32_t odd = (u >> 20) & 1u;
+    u += ((uint32_t)(7 - 127) << 23) + 0x7ffffu + odd;   // re-bias and round mantissa to 3 bits
+    r = u >> 20;
+  }
+  return r | sign;
+}
+
+__device__ __forceinline__ float e4m3_bits_to_f32(uint32_t b) {
+  uint32_t sign = (b & 0x80u) << 24;
+  uint32_t em = b & 0x7fu;
+  float v;
+  if (em == 0x7fu) {
+    v = __uint_as_float(0x7fc00000u);
+  } else if (em < 8u) {
+    v = (float)em * 0.001953125f;  // subnormal: m * 2^-9
+  } else {
+    v = __uint_as_float((em << 20) + ((uint32_t)(127 - 7) << 23));
+  }
+  return __uint_as_float(__float_as_uint(v) | sign);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// tanh-GELU in fp32: 0.5*x*(1 + tanh(u)), u = sqrt(2/pi)*(x + 0.044715 x^3), evaluated as
+// x / (1 + exp(-2u)), which is the same function without the cancellation in 1 + tanh(u).
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+  const float kBeta = 0.7978845608028654f;  // sqrt(2/pi)
+  const float kKappa = 0.044715f;
+  float u = kBeta * (x + kKappa * x * x * x);
+  float e = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);  // exp(-2u)
+  return x / (1.0f + e);
+}
+
+}  // namespace dsx

@@ -1,0 +1,324 @@
+// Bandwidth-bound row kernels of the DiT block: AdaLN modulate (LayerNorm + scale/shift),
+// gated residual, tanh-GELU, flow-match Euler update.  One workgroup of 256 threads owns one
+// row, keeps it in registers (16-byte loads, 8 bf16 per chunk), reduces through the wavefront
+// and a 4-entry LDS exchange, and can emit the row as bf16 and/or as per-token-scaled e4m3
+// (the operand format of the following FP8 GEMM) in the same pass.
+#include "common.h"
+
+namespace dsx {
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6;
+  __syncthreads();  // protect `red` against a previous reduction still being read
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__device__ __forceinline__ void unpack8(const u32x4& w, float* v) {
+  v[0] = bf16_lo(w.x); v[1] = bf16_hi(w.x); v[2] = bf16_lo(w.y); v[3] = bf16_hi(w.y);
+  v[4] = bf16_lo(w.z); v[5] = bf16_hi(w.z); v[6] = bf16_lo(w.w); v[7] = bf16_hi(w.w);
+}
+__device__ __forceinline__ u32x4 pack8(const float* v) {
+  u32x4 o;
+  o.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+  o.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+  o.z = f32_to_bf16_bits(v[4]) | (f32_to_bf16_bits(v[5]) << 16);
+  o.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
+  return o;
+}
+__device__ __forceinline__ u32x2 quant8(const float* v, float s) {
+  uint32_t b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) b[i] = f32_to_e4m3_bits(v[i] / s);
+  u32x2 r;
+  r.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+  r.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+  return r;
+}
+
+// Emit a row held as NCH register chunks of 8 already-bf16-rounded floats.
+template <int NCH>
+__device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint16_t* y, uint8_t* q,
+                                         float* q_scale, int64_t row, float* red) {
+  const int tid = threadIdx.x;
+  if (y) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = tid + i * 256;
+      if (c < nchunk) reinterpret_cast<u32x4*>(y)[c] = pack8(val[i]);
+    }
+  }
+  if (q) {
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = tid + i * 256;
+      if (c < nchunk) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(val[i][j]));
+      }
+    }
+    amax = block_max(amax, red);
+    const float s = fmaxf(amax, 1e-12f) / 448.0f;
+    if (tid == 0) q_scale[row] = s;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = tid + i * 256;
+      if (c < nchunk) reinterpret_cast<u32x2*>(q)[c] = quant8(val[i], s);
+    }
+  }
+}
+
+template <int NCH>
+__global__ __launch_bounds__(256) void adaln_modulate_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ scale,
+    const uint16_t* __restrict__ shift, int64_t mod_sb, int64_t rows_per_batch,
+    const uint16_t* __restrict__ ln_w, const uint16_t* __restrict__ ln_b, float eps,
+    uint16_t* __restrict__ y, int64_t ldy, uint8_t* __restrict__ q, int64_t ldq,
+    float* __restrict__ q_scale, int D) {
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const int nchunk = D >> 3;
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  float val[NCH][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = tid + i * 256;
+    if (c < nchunk) {
+      u32x4 w = xr[c];
+      unpack8(w, val[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += val[i][j];
+    }
+  }
+  const float mean = block_sum(sum, red) / (float)D;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = tid + i * 256;
+    if (c < nchunk) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float d = val[i][j] - mean;
+        sq += d * d;
+      }
+    }
+  }
+  const float rstd = rsqrtf(block_sum(sq, red) / (float)D + eps);
+  const int64_t bidx = row / rows_per_batch;
+  const u32x4* sc = scale ? reinterpret_cast<const u32x4*>(scale + bidx * mod_sb) : nullptr;
+  const u32x4* sh = shift ? reinterpret_cast<const u32x4*>(shift + bidx * mod_sb) : nullptr;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = tid + i * 256;
+    if (c < nchunk) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (val[i][j] - mean) * rstd;
+      if (ln_w) {
+        float w[8];
+        unpack8(reinterpret_cast<const u32x4*>(ln_w)[c], w);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] *= w[j];
+      }
+      if (ln_b) {
+        float bb[8];
+        unpack8(reinterpret_cast<const u32x4*>(ln_b)[c], bb);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] += bb[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j]);  // LayerNorm output tensor (bf16)
+      if (sc) {
+        float s8[8];
+        unpack8(sc[c], s8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j] * round_bf16(1.0f + s8[j]));
+      }
+      if (sh) {
+        float h8[8];
+        unpack8(sh[c], h8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j] + h8[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) val[i][j] = v[j];
+    }
+  }
+  emit_row<NCH>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
+                red);
+}
+
+template <int NCH>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                        uint16_t* __restrict__ y, int64_t ldy,
+                                                        uint8_t* __restrict__ q, int64_t ldq,
+                                                        float* __restrict__ q_scale, int D) {
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const int nchunk = D >> 3;
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  float val[NCH][8];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = tid + i * 256;
+    if (c < nchunk) {
+      u32x4 w = __builtin_nontemporal_load(xr + c);
+      unpack8(w, val[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(gelu_tanh_f32(val[i][j]));
+    }
+  }
+  emit_row<NCH>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
+                red);
+}
+
+__global__ __launch_bounds__(256) void gated_residual_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ yv, int64_t ldy,
+    const uint16_t* __restrict__ gate, int64_t gate_sb, int64_t rows_per_batch,
+    uint16_t* __restrict__ out, int64_t ldo, int64_t rows, int D) {
+  const int nchunk = D >> 3;
+  const int64_t total = rows * nchunk;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; id < total; id += stride) {
+    const int64_t row = id / nchunk;
+    const int c = (int)(id - row * nchunk);
+    float a[8], b[8];
+    unpack8(*reinterpret_cast<const u32x4*>(x + row * ldx + c * 8), a);
+    unpack8(*reinterpret_cast<const u32x4*>(yv + row * ldy + c * 8), b);
+    if (gate) {
+      float gt[8];
+      unpack8(*reinterpret_cast<const u32x4*>(gate + (row / rows_per_batch) * gate_sb + c * 8), gt);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) b[j] = round_bf16(gt[j] * b[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a[j] = a[j] + b[j];
+    *reinterpret_cast<u32x4*>(out + row * ldo + c * 8) = pack8(a);
+  }
+}
+
+template <bool FP32>
+__global__ __launch_bounds__(256) void euler_step_kernel(const void* __restrict__ lat,
+                                                         const void* __restrict__ v, float dt,
+                                                         void* __restrict__ out, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    if (FP32) {
+      const float a = reinterpret_cast<const float*>(lat)[i];
+      const float b = reinterpret_cast<const float*>(v)[i];
+      reinterpret_cast<float*>(out)[i] = __fadd_rn(a, __fmul_rn(b, dt));
+    } else {
+      const float a = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(lat)[i]);
+      const float b = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(v)[i]);
+      // `model_outputs * dt` is a bf16 tensor, the sum is taken in fp32 and rounded once
+      const float prod = round_bf16(__fmul_rn(b, dt));
+      reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_bf16_bits(__fadd_rn(a, prod));
+    }
+  }
+}
+
+static inline bool misaligned16(const void* p) { return ((uintptr_t)p & 15) != 0; }
+
+}  // namespace dsx
+
+extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale, const void* shift,
+                                  int64_t mod_sb, int64_t rows_per_batch, const void* ln_w,
+                                  const void* ln_b, float eps, void* y, int64_t ldy, void* q,
+                                  int64_t ldq, float* q_scale, int64_t rows, int64_t D,
+                                  void* stream) {
+  using namespace dsx;
+  if (!x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
+  if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || (y && ldy < D) || (q && ldq < D) ||
+      rows_per_batch <= 0)
+    return DSX_EBADSHAPE;
+  if ((ldx & 7) || (y && (ldy & 7)) || (q && (ldq & 7)) || (mod_sb & 7) || misaligned16(x) ||
+      misaligned16(y) || ((uintptr_t)q & 7) || misaligned16(scale) || misaligned16(shift) ||
+      misaligned16(ln_w) || misaligned16(ln_b))
+    return DSX_EALIGN;
+  if (rows == 0) return DSX_OK;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)rows), block(256);
+#define DSX_LAUNCH_ADALN(NCH)                                                                     \
+  adaln_modulate_kernel<NCH><<<grid, block, 0, st>>>(                                             \
+      (const uint16_t*)x, ldx, (const uint16_t*)scale, (const uint16_t*)shift, mod_sb,            \
+      rows_per_batch, (const uint16_t*)ln_w, (const uint16_t*)ln_b, eps, (uint16_t*)y, ldy,       \
+      (uint8_t*)q, ldq, q_scale, (int)D)
+  if (D <= 2048 * 2) DSX_LAUNCH_ADALN(2);
+  else if (D <= 2048 * 3) DSX_LAUNCH_ADALN(3);
+  else DSX_LAUNCH_ADALN(8);
+#undef DSX_LAUNCH_ADALN
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
+                             float* q_scale, int64_t rows, int64_t D, void* stream) {
+  using namespace dsx;
+  if (!x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
+  if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || (y && ldy < D) || (q && ldq < D))
+    return DSX_EBADSHAPE;
+  if ((ldx & 7) || (y && (ldy & 7)) || (q && (ldq & 7)) || misaligned16(x) || misaligned16(y) ||
+      ((uintptr_t)q & 7))
+    return DSX_EALIGN;
+  if (rows == 0) return DSX_OK;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)rows), block(256);
+#define DSX_LAUNCH_GELU(NCH)                                                                  \
+  gelu_tanh_kernel<NCH><<<grid, block, 0, st>>>((const uint16_t*)x, ldx, (uint16_t*)y, ldy,   \
+                                                (uint8_t*)q, ldq, q_scale, (int)D)
+  if (D <= 2048 * 2) DSX_LAUNCH_GELU(2);
+  else if (D <= 2048 * 6) DSX_LAUNCH_GELU(6);
+  else DSX_LAUNCH_GELU(8);
+#undef DSX_LAUNCH_GELU
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int dsx_gated_residual(const void* x, int64_t ldx, const void* y, int64_t ldy,
+                                  const void* gate, int64_t gate_sb, int64_t rows_per_batch,
+                                  void* out, int64_t ldo, int64_t rows, int64_t D, void* stream) {
+  using namespace dsx;
+  if (!x || !y || !out) return DSX_ENULL;
+  if (rows < 0 || D <= 0 || (D & 7) || D > (1 << 24) || ldx < D || ldy < D || ldo < D ||
+      rows_per_batch <= 0)
+    return DSX_EBADSHAPE;
+  if ((ldx & 7) || (ldy & 7) || (ldo & 7) || (gate_sb & 7) || misaligned16(x) || misaligned16(y) ||
+      misaligned16(out) || misaligned16(gate))
+    return DSX_EALIGN;
+  if (rows == 0) return DSX_OK;
+  const int64_t total = rows * (D >> 3);
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  gated_residual_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+      (const uint16_t*)x, ldx, (const uint16_t*)y, ldy, (const uint16_t*)gate, gate_sb,
+      rows_per_batch, (uint16_t*)out, ldo, rows, (int)D);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int dsx_flow_match_euler_step(const void* latents, const void* v, float dt, void* out,
+                                         int64_t n, int is_fp32, void* stream) {
+  using namespace dsx;
+  if (!latents || !v || !out) return DSX_ENULL;
+  if (n < 0) return DSX_EBADSHAPE;
+  if (n == 0) return DSX_OK;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipStream_t st = (hipStream_t)stream;
+  if (is_fp32)
+    euler_step_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(latents, v, dt, out, n);
+  else
+    euler_step_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(latents, v, dt, out, n);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}

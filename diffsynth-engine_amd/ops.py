@@ -1,0 +1,332 @@
+"""Tensor-level wrappers of the C-ABI kernels.
+
+PyTorch is used for device memory and the current stream only; every function below launches
+hand-written gfx950 kernels from libdsx.so on ``torch.cuda.current_stream()`` and raises if the
+library is missing or the tensors are not on a GPU.
+"""
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+FP8 = torch.float8_e4m3fn
+_BF16 = torch.bfloat16
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("diffsynth_engine_amd kernels need tensors on an MI355X device, got %s" % t.device)
+
+
+def _rows_2d(x: torch.Tensor) -> Tuple[torch.Tensor, int]:
+    """View x as (rows, D) with unit stride in the last dim; returns the view and its row stride."""
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    D = x.shape[-1]
+    if x.dim() == 2:
+        return x, x.stride(0)
+    x2 = x.reshape(-1, D) if x.is_contiguous() else None
+    if x2 is None:
+        # a column slice of a contiguous (…, Dfull) buffer keeps a uniform row stride
+        ld = x.stride(-2)
+        ok = all(x.stride(i) == x.stride(i + 1) * x.shape[i + 1] for i in range(x.dim() - 2))
+        if not ok:
+            x = x.contiguous()
+            return x.reshape(-1, D), D
+        x2 = x.as_strided((x.numel() // D, D), (ld, 1), x.storage_offset())
+        return x2, ld
+    return x2, D
+
+
+def quantize_fp8(x: torch.Tensor, scaled: bool = True):
+    """bf16 (…,K) -> (e4m3 (…,K), per-row fp32 scales or None).
+
+    ``scaled=False`` is the reference's bare ``input.to(torch.float8_e4m3fn)``
+    (diffsynth_engine/utils/fp8_linear.py:35); ``scaled=True`` divides each row by absmax/448 first.
+    """
+    _require_cuda(x)
+    if x.dtype != _BF16:
+        raise ValueError("quantize_fp8 expects bf16, got %s" % x.dtype)
+    x2, ldx = _rows_2d(x)
+    M, K = x2.shape
+    q = torch.empty((M, K), dtype=FP8, device=x.device)
+    scale = torch.empty((M,), dtype=torch.float32, device=x.device) if scaled else None
+    rc = _lib.load().dsx_quant_fp8_rowwise(_ptr(x2), ldx, _ptr(q), K, _ptr(scale), M, K, _stream())
+    _lib.check(rc, "dsx_quant_fp8_rowwise")
+    return q.view(*x.shape[:-1], K), scale
+
+
+def quantize_weight_fp8(w: torch.Tensor, scaled: bool = True):
+    """Weight cast of enable_fp8_linear (fp8_linear.py:15): returns (e4m3 weight, 0-dim fp32 scale or None)."""
+    _require_cuda(w)
+    if w.dtype not in (_BF16, torch.float32):
+        w = w.to(_BF16)
+    w = w.contiguous()
+    lib = _lib.load()
+    is_fp32 = int(w.dtype == torch.float32)
+    scale = None
+    if scaled:
+        amax = torch.zeros((), dtype=torch.float32, device=w.device)
+        _lib.check(lib.dsx_absmax(_ptr(w), w.numel(), is_fp32, _ptr(amax), _stream()), "dsx_absmax")
+        scale = torch.clamp(amax, min=1e-12) / 448.0
+    q = torch.empty(w.shape, dtype=FP8, device=w.device)
+    _lib.check(lib.dsx_cast_fp8_scaled(_ptr(w), is_fp32, _ptr(scale), _ptr(q), w.numel(), _stream()),
+               "dsx_cast_fp8_scaled")
+    return q, scale
+
+
+def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor] = None,
+             w_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3."""
+    _require_cuda(a_q, w_q)
+    if a_q.dtype != FP8 or w_q.dtype != FP8:
+        raise ValueError("fp8_gemm expects float8_e4m3fn operands")
+    if a_q.dim() != 2 or w_q.dim() != 2 or a_q.shape[1] != w_q.shape[1]:
+        raise ValueError("fp8_gemm shape mismatch: a %s, w %s" % (tuple(a_q.shape), tuple(w_q.shape)))
+    if a_q.stride(1) != 1:
+        a_q = a_q.contiguous()
+    if w_q.stride(1) != 1:
+        w_q = w_q.contiguous()
+    M, K = a_q.shape
+    N = w_q.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=_BF16, device=a_q.device)
+    elif out.dtype != _BF16 or out.shape != (M, N) or out.stride(1) != 1:
+        raise ValueError("fp8_gemm: bad `out`")
+    if bias is not None:
+        if bias.dtype != _BF16:
+            bias = bias.to(_BF16)
+        bias = bias.contiguous()
+    if a_scale is not None:
+        a_scale = a_scale.contiguous()
+    rc = _lib.load().dsx_fp8_gemm(_ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale), _ptr(w_scale),
+                                  _ptr(bias), _ptr(out), out.stride(0), M, N, K, _stream())
+    _lib.check(rc, "dsx_fp8_gemm")
+    return out
+
+
+def _bhsd_strides(t: torch.Tensor):
+    if t.stride(3) != 1:
+        raise ValueError("attention operands need unit stride in the head dim")
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def rope_table_from_freqs(freqs: torch.Tensor) -> torch.Tensor:
+    """Reference RoPE table (B,1,S,64,2,2) [[c,-s],[s,c]] (transformer_helper.py:54-64) -> (B,S,64,2) (c,s) fp32."""
+    if freqs.dim() != 6 or freqs.shape[-2:] != (2, 2):
+        raise ValueError("expected a (B,1,S,P,2,2) rotary table")
+    return torch.stack((freqs[:, 0, :, :, 0, 0], freqs[:, 0, :, :, 1, 0]), dim=-1).float().contiguous()
+
+
+def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float] = None,
+                   rope: Optional[torch.Tensor] = None, q_norm_w=None, k_norm_w=None, q2_norm_w=None,
+                   k2_norm_w=None, eps: float = 1e-6, out: Optional[torch.Tensor] = None,
+                   out2: Optional[torch.Tensor] = None):
+    """softmax(q k^T * scale) v over the concatenation [segment 1, segment 2] of rows.
+
+    q, k, v: (B,H,S,128) bf16 views with unit stride in the last dim (any other strides).
+    q2/k2/v2: optional second segment (same strides as the first), appended after the first.
+    rope: optional (B or 1, Sq, 64, 2) fp32 (cos, sin) table applied in-kernel to q and k;
+    *_norm_w: optional (128,) bf16 RMSNorm weights applied in-kernel before RoPE.
+    Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).
+    """
+    _require_cuda(q, k, v)
+    for t in (q, k, v, q2, k2, v2):
+        if t is not None and t.dtype != _BF16:
+            raise ValueError("attention expects bf16 tensors, got %s" % t.dtype)
+    B, H, S1, D = q.shape
+    if D != 128:
+        raise ValueError("head_dim must be 128, got %d" % D)
+    P = _lib.AttnParams()
+    S2 = 0 if q2 is None else q2.shape[2]
+    Skv1 = k.shape[2]
+    Skv2 = 0 if k2 is None else k2.shape[2]
+    if out is None:
+        out = torch.empty((B, S1, H, D), dtype=_BF16, device=q.device).transpose(1, 2)
+    if q2 is not None and out2 is None:
+        out2 = torch.empty((B, S2, H, D), dtype=_BF16, device=q.device).transpose(1, 2)
+
+    def same(a, b2, what):
+        if b2 is not None and _bhsd_strides(a) != _bhsd_strides(b2):
+            raise ValueError("both %s segments must share strides" % what)
+
+    same(q, q2, "q"); same(k, k2, "k"); same(v, v2, "v"); same(out, out2, "out")
+    P.q[0], P.q[1] = _ptr(q), _ptr(q2)
+    P.k[0], P.k[1] = _ptr(k), _ptr(k2)
+    P.v[0], P.v[1] = _ptr(v), _ptr(v2)
+    P.o[0], P.o[1] = _ptr(out), _ptr(out2)
+    P.sq[0], P.sq[1] = S1, S2
+    P.skv[0], P.skv[1] = Skv1, Skv2
+    P.q_sb, P.q_sh, P.q_ss = _bhsd_strides(q)
+    P.k_sb, P.k_sh, P.k_ss = _bhsd_strides(k)
+    P.v_sb, P.v_sh, P.v_ss = _bhsd_strides(v)
+    P.o_sb, P.o_sh, P.o_ss = _bhsd_strides(out)
+    P.batch, P.heads, P.head_dim = B, H, D
+    P.softmax_scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
+    keep = []
+    if rope is not None:
+        if rope.dtype != torch.float32 or rope.dim() != 4 or rope.shape[1:] != (S1 + S2, 64, 2):
+            raise ValueError("rope table must be fp32 (B|1, Sq, 64, 2)")
+        rope = rope.contiguous()
+        keep.append(rope)
+        P.rope = _ptr(rope)
+        P.rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
+    for i, (qw, kw) in enumerate(((q_norm_w, k_norm_w), (q2_norm_w, k2_norm_w))):
+        for name, w in (("q_norm_w", qw), ("k_norm_w", kw)):
+            if w is not None:
+                w = w.to(_BF16).contiguous()
+                keep.append(w)
+                getattr(P, name)[i] = _ptr(w)
+    P.norm_eps = eps
+    rc = _lib.load().dsx_attn_fwd(P, _stream())
+    _lib.check(rc, "dsx_attn_fwd")
+    return (out, out2) if q2 is not None else out
+
+
+def rmsnorm_rope(x: torch.Tensor, norm_w: Optional[torch.Tensor], rope: Optional[torch.Tensor], pos0: int = 0,
+                 eps: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMSNorm (per head, 128) then RoPE of a (B,H,S,128) bf16 view; returns a dense (B,H,S,128) tensor."""
+    _require_cuda(x)
+    B, H, S, D = x.shape
+    if D != 128 or x.dtype != _BF16:
+        raise ValueError("rmsnorm_rope expects bf16 (B,H,S,128)")
+    if out is None:
+        out = torch.empty((B, H, S, D), dtype=_BF16, device=x.device)
+    if norm_w is not None:
+        norm_w = norm_w.to(_BF16).contiguous()
+    rope_sb = 0
+    if rope is not None:
+        rope = rope.contiguous()
+        rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
+    xs, os_ = _bhsd_strides(x), _bhsd_strides(out)
+    rc = _lib.load().dsx_rmsnorm_rope(_ptr(x), xs[0], xs[1], xs[2], _ptr(norm_w), eps, _ptr(rope), rope_sb, pos0,
+                                      _ptr(out), os_[0], os_[1], os_[2], B, H, S, _stream())
+    _lib.check(rc, "dsx_rmsnorm_rope")
+    return out
+
+
+def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Optional[torch.Tensor],
+                   eps: float = 1e-6, ln_weight=None, ln_bias=None, want_bf16: bool = True,
+                   want_fp8: bool = False):
+    """LayerNorm(x) * (1 + scale) + shift per token; x (B,S,D) bf16, scale/shift (B,D) or (B,1,D) bf16.
+
+    Returns y (bf16) and/or (q e4m3, q_scale fp32 per token) depending on want_*.
+    """
+    _require_cuda(x)
+    if x.dtype != _BF16:
+        raise ValueError("adaln_modulate expects bf16")
+    shp = x.shape
+    D = shp[-1]
+    B = shp[0] if x.dim() == 3 else 1
+    x2, ldx = _rows_2d(x)
+    rows = x2.shape[0]
+    mod_sb = 0
+
+    def prep(t):
+        nonlocal mod_sb
+        if t is None:
+            return None
+        t = t.reshape(-1, D)  # a view for (B,D), (B,1,D) and chunk() slices of a (B,k*D) projection
+        if t.stride(1) != 1:
+            t = t.contiguous()
+        if t.shape[0] not in (1, B):
+            raise ValueError("modulation must have one row per batch entry")
+        sb = t.stride(0) if t.shape[0] > 1 else 0
+        if mod_sb and sb and mod_sb != sb:
+            raise ValueError("scale and shift must share a batch stride")
+        mod_sb = sb or mod_sb
+        return t
+
+    scale_t, shift_t = prep(scale), prep(shift)
+    y = torch.empty((rows, D), dtype=_BF16, device=x.device) if want_bf16 else None
+    q = torch.empty((rows, D), dtype=FP8, device=x.device) if want_fp8 else None
+    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
+    rc = _lib.load().dsx_adaln_modulate(_ptr(x2), ldx, _ptr(scale_t), _ptr(shift_t), mod_sb, max(rows // B, 1),
+                                        _ptr(ln_weight), _ptr(ln_bias), eps, _ptr(y), D, _ptr(q), D, _ptr(qs), rows,
+                                        D, _stream())
+    _lib.check(rc, "dsx_adaln_modulate")
+    res = []
+    if want_bf16:
+        res.append(y.view(shp))
+    if want_fp8:
+        res += [q.view(shp), qs]
+    return res[0] if len(res) == 1 else tuple(res)
+
+
+def gated_residual(x: torch.Tensor, y: torch.Tensor, gate: Optional[torch.Tensor],
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x + gate * y (gate (B,D) / (B,1,D) or None); bf16, rounding bf16(x + bf16(gate*y))."""
+    _require_cuda(x, y)
+    shp = x.shape
+    D = shp[-1]
+    B = shp[0] if x.dim() == 3 else 1
+    x2, ldx = _rows_2d(x)
+    y2, ldy = _rows_2d(y)
+    rows = x2.shape[0]
+    gate_sb = 0
+    if gate is not None:
+        gate = gate.reshape(-1, D)
+        if gate.stride(1) != 1:
+            gate = gate.contiguous()
+        gate_sb = gate.stride(0) if gate.shape[0] > 1 else 0
+    if out is None:
+        out = torch.empty((rows, D), dtype=_BF16, device=x.device)
+        o2, ldo = out, D
+    else:
+        o2, ldo = _rows_2d(out)
+    rc = _lib.load().dsx_gated_residual(_ptr(x2), ldx, _ptr(y2), ldy, _ptr(gate), gate_sb, max(rows // B, 1),
+                                        _ptr(o2), ldo, rows, D, _stream())
+    _lib.check(rc, "dsx_gated_residual")
+    return out.view(shp)
+
+
+def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, out: Optional[torch.Tensor] = None):
+    """tanh-GELU over the last dim of a bf16 tensor (a column slice of a wider buffer is fine)."""
+    _require_cuda(x)
+    if x.dtype != _BF16:
+        raise ValueError("gelu_tanh expects bf16")
+    shp = x.shape
+    D = shp[-1]
+    x2, ldx = _rows_2d(x)
+    rows = x2.shape[0]
+    y, ldy = None, D
+    if want_bf16:
+        if out is not None:
+            y, ldy = _rows_2d(out)
+        else:
+            y = torch.empty((rows, D), dtype=_BF16, device=x.device)
+    q = torch.empty((rows, D), dtype=FP8, device=x.device) if want_fp8 else None
+    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
+    rc = _lib.load().dsx_gelu_tanh(_ptr(x2), ldx, _ptr(y), ldy, _ptr(q), D, _ptr(qs), rows, D, _stream())
+    _lib.check(rc, "dsx_gelu_tanh")
+    res = []
+    if want_bf16:
+        res.append(out if out is not None else y.view(shp))
+    if want_fp8:
+        res += [q.view(shp), qs]
+    return res[0] if len(res) == 1 else tuple(res)
+
+
+def flow_match_euler_step(latents: torch.Tensor, model_outputs: torch.Tensor, dt: float) -> torch.Tensor:
+    """latents + model_outputs * dt in fp32, cast back (flow_match_euler.py:11-19)."""
+    _require_cuda(latents, model_outputs)
+    if latents.dtype != model_outputs.dtype or latents.dtype not in (_BF16, torch.float32):
+        raise ValueError("flow_match_euler_step expects matching bf16 or fp32 tensors")
+    a, b = latents.contiguous(), model_outputs.contiguous()
+    out = torch.empty_like(a)
+    rc = _lib.load().dsx_flow_match_euler_step(_ptr(a), _ptr(b), float(dt), _ptr(out), a.numel(),
+                                               int(a.dtype == torch.float32), _stream())
+    _lib.check(rc, "dsx_flow_match_euler_step")
+    return out

@@ -1,0 +1,181 @@
+/*
+ * dsx.h — C ABI of libdsx.so: hand-written gfx950 (MI355X / CDNA4) kernels for the
+ * DiT denoising-step hot path of DiffSynth-Engine.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller unless stated otherwise;
+ *     the library never allocates, frees or keeps device memory;
+ *   - every launch goes to the hipStream_t passed as `stream` (NULL = default stream)
+ *     and returns without synchronising;
+ *   - the return value is DSX_OK (0) or a negative DSX_E* code; nothing throws or exits;
+ *   - "bf16" is the 16-bit brain float, "e4m3" the 8-bit OCP float8_e4m3fn
+ *     (bias 7, max 448, no inf, 0x7f/0xff = NaN);
+ *   - strides and leading dimensions are counted in ELEMENTS of the tensor they describe.
+ *
+ * Each entry point names the interface of the reference (DiffSynth-Engine v0.1.1,
+ * paths relative to its root) whose arithmetic it replaces.
+ */
+#ifndef DSX_H
+#define DSX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DSX_ABI_VERSION 1
+
+enum {
+  DSX_OK = 0,
+  DSX_EBADSHAPE = -1, /* a size/stride the kernels do not support          */
+  DSX_EALIGN = -2,    /* a pointer or leading dimension not 16-byte aligned */
+  DSX_EARCH = -3,     /* current device is not gfx950                       */
+  DSX_ELAUNCH = -4,   /* hipLaunchKernel reported an error                  */
+  DSX_ENULL = -5      /* a required pointer is NULL                         */
+};
+
+/* Version of this ABI (DSX_ABI_VERSION of the library that was built). */
+int dsx_abi_version(void);
+
+/* Static, NUL-terminated description of a DSX_* code. */
+const char* dsx_strerror(int code);
+
+/* 0 when the current HIP device is gfx950, DSX_EARCH otherwise. */
+int dsx_check_device(void);
+
+/*
+ * Activation quantisation: bf16 -> e4m3, one row ("token") at a time.
+ * Replaces `input.to(torch.float8_e4m3fn)` in diffsynth_engine/utils/fp8_linear.py:35.
+ *
+ *   scale_out == NULL : bare cast, q[m,k] = e4m3_rne(x[m,k]); exactly torch's cast
+ *                       (round-to-nearest-even, subnormals kept, |v| > 464 -> NaN).
+ *   scale_out != NULL : dynamic per-token scale, s[m] = max(absmax(x[m,:]), 1e-12) / 448
+ *                       (fp32 division), q[m,k] = e4m3_rne(float(x[m,k]) / s[m]).
+ * x: (M,K) bf16, row stride ldx; q: (M,K) e4m3, row stride ldq; K % 8 == 0.
+ */
+int dsx_quant_fp8_rowwise(const void* x, int64_t ldx, void* q, int64_t ldq, float* scale_out,
+                          int64_t M, int64_t K, void* stream);
+
+/*
+ * Weight quantisation helper: fp32 absmax of a bf16 (or fp32 when is_fp32 != 0) buffer of n
+ * elements into *absmax_out (device fp32, must be zero-initialised by the caller).
+ * Used by enable_fp8_linear (diffsynth_engine/utils/fp8_linear.py:7-17) for the per-tensor scale.
+ */
+int dsx_absmax(const void* x, int64_t n, int is_fp32, float* absmax_out, void* stream);
+
+/*
+ * Per-tensor scaled cast: q[i] = e4m3_rne(float(x[i]) / *scale) (scale == NULL: bare cast).
+ * Replaces `module.weight.data.to(torch.float8_e4m3fn)` (fp8_linear.py:15).
+ */
+int dsx_cast_fp8_scaled(const void* x, int is_fp32, const float* scale, void* q, int64_t n,
+                        void* stream);
+
+/*
+ * FP8 scaled GEMM with fused bias:
+ *   out[m,n] = bf16( (sum_k a[m,k] * w[n,k]) * a_scale[m] * (*w_scale) + bias[n] ), fp32 accumulate.
+ * Replaces `torch._scaled_mm(input, weight.T, scale_a, scale_b, bias, out_dtype)` in
+ * diffsynth_engine/utils/fp8_linear.py:41-48,52-59.
+ *   a: (M,K) e4m3 row-major (lda); w: (N,K) e4m3 row-major (ldw), i.e. nn.Linear.weight as stored;
+ *   a_scale: M fp32 or NULL (= 1); w_scale: device fp32 scalar or NULL (= 1); bias: N bf16 or NULL;
+ *   out: (M,N) bf16 (ldo).  K % 16 == 0, lda/ldw % 16 == 0, ldo % 8 == 0 when N % 8 == 0.
+ */
+int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t ldw, const float* a_scale,
+                 const float* w_scale, const void* bias, void* out, int64_t ldo, int64_t M,
+                 int64_t N, int64_t K, void* stream);
+
+/*
+ * Flash attention, head dim 128, bf16 in/out, fp32 online softmax, non-causal, no mask.
+ * Replaces `_attn_func(q, k, v)` = F.scaled_dot_product_attention in
+ * diffsynth_engine/models/flux/flux_dit.py:21,182,267,303 and `attention()` in
+ * diffsynth_engine/models/wan/wan_dit.py:18-22; with `rope`/`*_norm_w` set it also replaces
+ * RMSNorm (models/basic/transformer_helper.py:73-78) and apply_rope (flux_dit.py:154-159)
+ * on q and k, and the text-first concat (flux_dit.py:176-178) through the two segments.
+ *
+ * The query sequence is the concatenation of up to two segments (segment 0 first), each read
+ * from its own base pointer with shared strides; likewise keys/values and the output.
+ * Element (b,h,s,d) of segment g of q lives at q[g][b*q_sb + h*q_sh + s*q_ss + d].
+ */
+typedef struct dsx_attn_params {
+  const void* q[2];   /* bf16; q[1] may be NULL when sq[1] == 0 */
+  const void* k[2];
+  const void* v[2];
+  void* o[2];         /* bf16 */
+  int64_t sq[2];      /* query rows per segment  */
+  int64_t skv[2];     /* key/value rows per segment */
+  int64_t q_sb, q_sh, q_ss;
+  int64_t k_sb, k_sh, k_ss;
+  int64_t v_sb, v_sh, v_ss;
+  int64_t o_sb, o_sh, o_ss;
+  int32_t batch, heads, head_dim; /* head_dim must be 128 */
+  float softmax_scale;            /* e.g. 1/sqrt(128) */
+  /* Optional fused pre-processing of q and k (NULL = off):
+   *   rope      : fp32 table (rope_sb*b + pos*128 + 2*i + {0,1}) = (cos, sin) of pair i at
+   *               joint position pos (segment 0 rows first); applied to q and k on pairs (2i,2i+1),
+   *               result rounded to bf16.
+   *   q_norm_w/k_norm_w[g] : bf16 (128,) RMSNorm weight of segment g; y = bf16(bf16(x*rsqrt(ms+eps))*w). */
+  const float* rope;
+  int64_t rope_sb;
+  const void* q_norm_w[2];
+  const void* k_norm_w[2];
+  float norm_eps;
+  int32_t reserved;
+} dsx_attn_params;
+
+int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
+
+/*
+ * Standalone RMSNorm + RoPE of q and k (same arithmetic and rounding points as the fused
+ * option of dsx_attn_fwd), written to a dense (B,H,S,128) bf16 buffer.  One tensor per call.
+ * Replaces RMSNorm.forward (transformer_helper.py:73-78) followed by apply_rope (flux_dit.py:154-159).
+ */
+int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss, const void* norm_w,
+                     float eps, const float* rope, int64_t rope_sb, int64_t rope_pos0, void* out,
+                     int64_t o_sb, int64_t o_sh, int64_t o_ss, int32_t batch, int32_t heads,
+                     int64_t seq, void* stream);
+
+/*
+ * AdaLN modulate: y = LayerNorm(x; eps, no affine) * (1 + scale) + shift, one row per token.
+ * Replaces `self.norm(x) * (1 + scale) + shift` in models/basic/transformer_helper.py:17,21,35,
+ * models/flux/flux_dit.py:228,233,334 and `modulate(norm(x), shift, scale)` in
+ * models/wan/wan_dit.py:25-26,188,191,236.
+ *   x: (B*S, D) bf16 (ldx); scale, shift: bf16 (D,) per batch entry, batch stride mod_sb
+ *   (row r uses batch r / rows_per_batch); ln_w/ln_b: optional bf16 affine (Wan norm3) or NULL.
+ *   y_bf16 (ldy) and/or (q_fp8 (ldq) + q_scale[rows]) are written; either may be NULL.
+ *   Rounding follows the bf16 op sequence: bf16(LN) -> bf16(1+scale) -> bf16(mul) -> bf16(add).
+ *   D % 8 == 0, D <= 16384.
+ */
+int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale, const void* shift,
+                       int64_t mod_sb, int64_t rows_per_batch, const void* ln_w, const void* ln_b,
+                       float eps, void* y, int64_t ldy, void* q, int64_t ldq, float* q_scale,
+                       int64_t rows, int64_t D, void* stream);
+
+/*
+ * Gated residual: out = x + gate * y  (gate == NULL: out = x + y), bf16, gate (D,) per batch entry.
+ * Replaces flux_dit.py:227,229,232,234,318-319 and wan_dit.py:189,190,192.
+ * Rounding: bf16(x + bf16(gate * y)).
+ */
+int dsx_gated_residual(const void* x, int64_t ldx, const void* y, int64_t ldy, const void* gate,
+                       int64_t gate_sb, int64_t rows_per_batch, void* out, int64_t ldo,
+                       int64_t rows, int64_t D, void* stream);
+
+/*
+ * tanh-GELU: y = bf16(gelu_tanh(float(x))).  Replaces nn.GELU(approximate="tanh")
+ * (flux_dit.py:209,215,315; wan_dit.py:180).  x may be a column slice of a wider buffer (ldx).
+ * y_bf16 and/or (q_fp8 + q_scale) are written as in dsx_adaln_modulate.  D % 8 == 0, D <= 16384.
+ */
+int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
+                  float* q_scale, int64_t rows, int64_t D, void* stream);
+
+/*
+ * Flow-match Euler update: out = cast(float(latents) + float(v) * dt), element-wise, bf16 or fp32
+ * (is_fp32 selects the storage type of all three buffers).
+ * Replaces FlowMatchEulerSampler.step (algorithm/sampler/flow_match/flow_match_euler.py:11-19).
+ */
+int dsx_flow_match_euler_step(const void* latents, const void* v, float dt, void* out, int64_t n,
+                              int is_fp32, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSX_H */

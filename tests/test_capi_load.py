@@ -1,0 +1,122 @@
+"""CPU-side checks of the drop-in boundary: the library loads, exports every declared symbol,
+and the host-side mirrors keep the reference's error conventions.  No kernel is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "dsx.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dsx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.SIGNATURES) == names  # the ctypes table and the header agree
+
+
+def test_abi_version_and_strerror():
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    assert lib.dsx_abi_version() == 1
+    assert _lib.strerror(0) == "ok"
+    for code in (-1, -2, -3, -4, -5):
+        assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
+    assert "unknown" in _lib.strerror(-99)
+
+
+def test_attn_params_struct_layout_matches_header():
+    from diffsynth_engine_amd import _lib
+
+    # 8 + 4 pointers/int64 pairs (12*8*... ) : q,k,v,o,sq,skv = 6*16; 12 strides*8; 3 int32 + float; rope, rope_sb;
+    # 2*16 norm pointers; float + int32
+    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 8 + 16 + 8 + 8 + 32 + 8
+
+
+def test_null_and_shape_errors_without_touching_the_gpu():
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    assert lib.dsx_fp8_gemm(None, 16, None, 16, None, None, None, None, 16, 16, 16, 16, None) == _lib.DSX_ENULL
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) & ~15
+    assert lib.dsx_fp8_gemm(p16, 24, p16, 24, None, None, None, p16, 16, 16, 16, 24, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_fp8_gemm(p16 + 1, 16, p16, 16, None, None, None, p16, 16, 16, 16, 16, None) == _lib.DSX_EALIGN
+    assert lib.dsx_quant_fp8_rowwise(p16, 12, p16, 12, None, 4, 12, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_attn_fwd(None, None) == _lib.DSX_ENULL
+    P = _lib.AttnParams()
+    P.head_dim, P.batch, P.heads = 64, 1, 1
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_gelu_tanh(p16, 8, None, 8, None, 8, None, 1, 8, None) == _lib.DSX_ENULL
+    assert lib.dsx_adaln_modulate(p16, 12, None, None, 0, 1, None, None, 1e-6, p16, 12, None, 0, None, 1, 12,
+                                  None) == _lib.DSX_EBADSHAPE
+    with pytest.raises(ValueError):
+        _lib.check(_lib.DSX_EALIGN, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.DSX_EARCH, "x")
+
+
+def test_missing_library_is_an_import_error(monkeypatch):
+    from diffsynth_engine_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libdsx.so")
+    with pytest.raises(ImportError):
+        _lib.load()
+
+
+def test_attention_name_validation_mirrors_reference():
+    """Unknown implementation names raise ValueError (flux_dit.py:483-486)."""
+    import types
+
+    from diffsynth_engine_amd import mi355x_attention, set_attn_implementation
+
+    with pytest.raises(ValueError):
+        set_attn_implementation("sage_attn_typo")
+    fake = types.SimpleNamespace(_attn_func=F.scaled_dot_product_attention)
+    set_attn_implementation("mi355x", flux_dit_module=fake)
+    assert fake._attn_func is mi355x_attention
+    set_attn_implementation("sdpa", flux_dit_module=fake)
+    assert fake._attn_func is F.scaled_dot_product_attention
+
+
+def test_cpu_tensors_are_refused_not_silently_computed():
+    from diffsynth_engine_amd import mi355x_attention, ops
+
+    q = torch.zeros(1, 1, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        mi355x_attention(q, q, q)
+    with pytest.raises(RuntimeError):
+        ops.quantize_fp8(torch.zeros(2, 16, dtype=torch.bfloat16))
+
+
+def test_fp8_inference_patches_and_restores_f_linear():
+    """Same observable behaviour as fp8_linear.py:20-64; additionally restores on exceptions."""
+    from diffsynth_engine_amd import fp8_inference
+    from diffsynth_engine_amd import fp8_linear as mod
+
+    orig = F.linear
+    with fp8_inference(False):
+        assert F.linear is orig
+    with fp8_inference():
+        assert F.linear is mod.fp8_linear
+    assert F.linear is orig
+    with pytest.raises(KeyError):
+        with fp8_inference(True):
+            raise KeyError("boom")
+    assert F.linear is orig

@@ -1,0 +1,151 @@
+"""GPU parity: flash attention (plain, joint two-segment, cross, fused RMSNorm+RoPE) vs the fp32 oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import dit_ops as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-2  # max |err| / max |ref|, the bar stated for the attention kernel
+
+
+def _rel_err(got, want):
+    return ((got.float() - want.float()).abs().max() / want.float().abs().max()).item()
+
+
+def _qkv(B, H, Sq, Skv, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, Sq, 128, generator=g).bfloat16()
+    k = torch.randn(B, H, Skv, 128, generator=g).bfloat16()
+    v = torch.randn(B, H, Skv, 128, generator=g).bfloat16()
+    return q, k, v
+
+
+@pytest.mark.parametrize("B,H,Sq,Skv", [(1, 2, 256, 64), (1, 1, 64, 256), (2, 3, 300, 300), (1, 2, 1, 1),
+                                        (1, 2, 1280, 1280), (1, 1, 520, 77), (1, 4, 33, 512)])
+def test_attention_matches_fp32_sdpa(dev, B, H, Sq, Skv):
+    from diffsynth_engine_amd import mi355x_attention
+
+    q, k, v = _qkv(B, H, Sq, Skv, seed=Sq * 7 + Skv)
+    want = O.sdpa(q.float(), k.float(), v.float())
+    got = mi355x_attention(q.to(dev), k.to(dev), v.to(dev)).cpu()
+    assert got.shape == want.shape and got.dtype == torch.bfloat16
+    assert _rel_err(got, want) <= TOL
+
+
+def test_attention_against_torch_sdpa_library(dev):
+    """Second opinion: torch's own fp32 SDPA (the routine the reference calls)."""
+    from diffsynth_engine_amd import mi355x_attention
+
+    q, k, v = _qkv(1, 2, 384, 384, seed=3)
+    want = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    got = mi355x_attention(q.to(dev), k.to(dev), v.to(dev)).cpu()
+    assert _rel_err(got, want) <= TOL
+
+
+def test_attention_noncontiguous_packed_qkv_views(dev):
+    """The views FluxJointAttention hands to the slot: (B,S,3H,D).transpose(1,2).chunk(3,1) (flux_dit.py:165-167)."""
+    from diffsynth_engine_amd import mi355x_attention
+
+    B, S, H = 1, 320, 3
+    qkv = torch.randn(B, S, 3 * H * 128, generator=torch.Generator().manual_seed(1)).bfloat16()
+    q, k, v = qkv.view(B, S, 3 * H, 128).transpose(1, 2).chunk(3, dim=1)
+    want = O.sdpa(q.float(), k.float(), v.float())
+    qd, kd, vd = qkv.to(dev).view(B, S, 3 * H, 128).transpose(1, 2).chunk(3, dim=1)
+    got = mi355x_attention(qd, kd, vd).cpu()
+    assert _rel_err(got, want) <= TOL
+
+
+def test_softmax_invariants(dev):
+    """Constant V => output equals that constant; permuting keys together with values changes nothing."""
+    from diffsynth_engine_amd import mi355x_attention
+
+    q, k, v = _qkv(1, 2, 200, 333, seed=9)
+    vc = torch.full_like(v, 0.75)
+    out = mi355x_attention(q.to(dev), k.to(dev), vc.to(dev)).cpu().float()
+    assert (out - 0.75).abs().max().item() <= 0.75 * 2 ** -7
+    perm = torch.randperm(333, generator=torch.Generator().manual_seed(2))
+    a = mi355x_attention(q.to(dev), k.to(dev), v.to(dev)).cpu().float()
+    b = mi355x_attention(q.to(dev), k[:, :, perm].contiguous().to(dev), v[:, :, perm].contiguous().to(dev)).cpu().float()
+    assert (a - b).abs().max().item() <= 2e-2
+
+
+def test_joint_two_segment_equals_concat(dev):
+    """Text-first joint attention from two base pointers == attention over torch.cat (flux_dit.py:176-178)."""
+    from diffsynth_engine_amd import ops
+
+    H, St, Si = 2, 72, 200
+    qt, kt, vt = _qkv(1, H, St, St, seed=11)
+    qi, ki, vi = _qkv(1, H, Si, Si, seed=12)
+    want = O.sdpa(torch.cat([qt, qi], 2).float(), torch.cat([kt, ki], 2).float(), torch.cat([vt, vi], 2).float())
+    o1, o2 = ops.attention_bhsd(qt.to(dev), kt.to(dev), vt.to(dev), q2=qi.to(dev), k2=ki.to(dev), v2=vi.to(dev))
+    got = torch.cat([o1.cpu(), o2.cpu()], dim=2)
+    assert _rel_err(got, want) <= TOL
+
+
+def _flux_ids(St, side):
+    txt = torch.zeros(1, St, 3)
+    img = torch.zeros(side, side, 3)
+    img[..., 1] += torch.arange(side)[:, None]
+    img[..., 2] += torch.arange(side)[None, :]
+    return torch.cat([txt, img.reshape(1, -1, 3)], dim=1)
+
+
+@pytest.mark.parametrize("wstd", [0.0, 0.1])
+def test_fused_rmsnorm_rope_joint_attention(dev, wstd):
+    """RMSNorm + 3-axis RoPE applied in-kernel == oracle RMSNorm -> concat -> apply_rope -> SDPA (flux_dit.py:161-183)."""
+    from diffsynth_engine_amd import ops
+
+    H, St, side = 2, 64, 12
+    Si = side * side
+    g = torch.Generator().manual_seed(21)
+    qt, kt, vt = _qkv(1, H, St, St, seed=13)
+    qi, ki, vi = _qkv(1, H, Si, Si, seed=14)
+    w = [(1.0 + wstd * torch.randn(128, generator=g)).bfloat16() for _ in range(4)]  # q_a, k_a, q_b, k_b
+    freqs = O.rope_table(_flux_ids(St, side), (16, 56, 56), 10000)
+    # oracle in bf16 (the reference's dtype) up to the attention inputs, fp32 attention
+    q = torch.cat([O.rms_norm(qt, w[2], 1e-6), O.rms_norm(qi, w[0], 1e-6)], dim=2)
+    k = torch.cat([O.rms_norm(kt, w[3], 1e-6), O.rms_norm(ki, w[1], 1e-6)], dim=2)
+    q, k = O.apply_rope(q, freqs), O.apply_rope(k, freqs)
+    want = O.sdpa(q.float(), k.float(), torch.cat([vt, vi], 2).float())
+    table = ops.rope_table_from_freqs(freqs).to(dev)
+    o1, o2 = ops.attention_bhsd(qt.to(dev), kt.to(dev), vt.to(dev), q2=qi.to(dev), k2=ki.to(dev), v2=vi.to(dev),
+                                rope=table, q_norm_w=w[2].to(dev), k_norm_w=w[3].to(dev), q2_norm_w=w[0].to(dev),
+                                k2_norm_w=w[1].to(dev))
+    got = torch.cat([o1.cpu(), o2.cpu()], dim=2)
+    assert _rel_err(got, want) <= TOL
+    # the standalone pre-pass must agree with the oracle's bf16 q almost bit for bit
+    qn = ops.rmsnorm_rope(qi.to(dev), w[0].to(dev), table, pos0=St).cpu()
+    ref = q[:, :, St:]
+    diff = (qn.float() - ref.float()).abs()
+    assert (diff > 0).float().mean().item() < 0.01  # rare 1-ulp flips from the rsqrt / sum order
+    assert diff.max().item() <= 2 ** -6 * ref.float().abs().max().item()
+
+
+def test_wan_seam_cross_attention(dev):
+    """wan_dit.attention contract (wan_dit.py:18-22): (B,S,H*D), Lq != Lk."""
+    from diffsynth_engine_amd import wan_attention
+
+    B, H, Sq, Skv = 1, 3, 250, 64
+    q, k, v = _qkv(B, H, Sq, Skv, seed=5)
+    want = O.sdpa(q.float(), k.float(), v.float()).transpose(1, 2).reshape(B, Sq, H * 128)
+    flat = lambda t: t.transpose(1, 2).reshape(B, t.shape[2], H * 128).contiguous()
+    got = wan_attention(flat(q).to(dev), flat(k).to(dev), flat(v).to(dev), H).cpu()
+    assert _rel_err(got, want) <= TOL
+
+
+def test_bshd_attention_entry_and_errors(dev):
+    from diffsynth_engine_amd import attention
+
+    q, k, v = _qkv(1, 2, 100, 100, seed=6)
+    want = O.sdpa(q.float(), k.float(), v.float()).transpose(1, 2)
+    got = attention(q.transpose(1, 2).contiguous().to(dev), k.transpose(1, 2).contiguous().to(dev),
+                    v.transpose(1, 2).contiguous().to(dev), attn_impl="mi355x").cpu()
+    assert _rel_err(got, want) <= TOL
+    with pytest.raises(ValueError):
+        attention(q, k, v, attn_impl="flash3")
+    with pytest.raises(ValueError):
+        bad = torch.zeros(1, 1, 8, 64, dtype=torch.bfloat16, device=dev)
+        attention(bad, bad, bad)

@@ -1,0 +1,129 @@
+"""GPU parity: e4m3 quantisation (bit-exact) and the FP8 scaled GEMM, through the C-ABI."""
+import pytest
+import torch
+
+from oracle import fp8 as ofp8
+
+pytestmark = pytest.mark.gpu
+
+
+def _all_bf16(dev):
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    return bits.view(torch.bfloat16).to(dev)
+
+
+def test_bare_cast_bit_exact_all_bf16(dev):
+    """Every bf16 bit pattern through the unscaled row quantiser == torch's cast (fp8_linear.py:35)."""
+    from diffsynth_engine_amd import ops
+
+    x = _all_bf16(dev).view(64, 1024)
+    q, s = ops.quantize_fp8(x, scaled=False)
+    assert s is None
+    want = x.cpu().to(torch.float8_e4m3fn)
+    got, want = q.cpu().view(torch.uint8), want.view(torch.uint8)
+    # NaN payload sign may differ only for NaN inputs; compare NaN-ness there, bits elsewhere
+    nan_in = torch.isnan(x.cpu().float())
+    assert torch.equal(got[~nan_in], want[~nan_in])
+    assert bool(((got[nan_in] & 0x7F) == 0x7F).all())
+
+
+@pytest.mark.parametrize("M,K", [(1, 64), (7, 3072), (130, 12288), (33, 4096), (5, 16384), (3, 8)])
+def test_rowwise_scaled_quant_bit_exact(dev, M, K):
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(M * 1000 + K)
+    x = torch.randn(M, K, generator=g)
+    x[:, :: max(K // 7, 1)] *= 20.0
+    if M > 2:
+        x[2] = 0.0  # all-zero row: scale clamps at 1e-12/448
+    x = x.bfloat16()
+    q, s = ops.quantize_fp8(x.to(dev), scaled=True)
+    wq, ws = ofp8.quantize_rowwise(x, scaled=True)
+    assert torch.equal(s.cpu(), ws)
+    assert torch.equal(q.cpu().view(torch.uint8), wq.view(torch.uint8))
+
+
+def test_rowwise_quant_strided_rows(dev):
+    from diffsynth_engine_amd import ops
+
+    x = torch.randn(16, 512).bfloat16()
+    xs = x.to(dev)[:, 128:384]
+    q, s = ops.quantize_fp8(xs, scaled=True)
+    wq, ws = ofp8.quantize_rowwise(x[:, 128:384], scaled=True)
+    assert torch.equal(s.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8), wq.view(torch.uint8))
+
+
+def test_weight_quant_matches_oracle(dev):
+    from diffsynth_engine_amd import ops
+
+    for dtype in (torch.bfloat16, torch.float32):
+        w = (torch.randn(300, 200) * 0.02).to(dtype)
+        q, s = ops.quantize_weight_fp8(w.to(dev), scaled=True)
+        wq, ws = ofp8.quantize_weight(w, scaled=True)
+        assert torch.equal(s.cpu(), ws)
+        assert torch.equal(q.cpu().view(torch.uint8), wq.view(torch.uint8))
+        q, s = ops.quantize_weight_fp8(w.to(dev), scaled=False)
+        assert s is None and torch.equal(q.cpu().view(torch.uint8), w.to(torch.float8_e4m3fn).view(torch.uint8))
+
+
+def _gemm_case(dev, M, N, K, seed, bias=True, scaled=True):
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(N, K, generator=g) * 0.02
+    x = torch.randn(M, K, generator=g)
+    x[:, torch.randperm(K, generator=g)[: max(K // 1000, 1)]] *= 20.0
+    x = x.bfloat16()
+    b = torch.randn(N, generator=g).bfloat16() if bias else None
+    wq, ws = ofp8.quantize_weight(w, scaled=scaled)
+    xq, xs = ofp8.quantize_rowwise(x, scaled=scaled)
+    want = ofp8.scaled_linear(xq, xs, wq, ws, b)
+    got = ops.fp8_gemm(xq.to(dev), wq.to(dev), None if xs is None else xs.to(dev),
+                       None if ws is None else ws.to(dev), None if b is None else b.to(dev)).cpu()
+    return got.float(), want.float()
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (256, 256, 3072), (512, 768, 256), (300, 200, 64),
+                                   (1000, 3072, 1024), (17, 64, 3072), (9, 264, 16), (257, 513, 144)])
+def test_fp8_gemm_matches_dequantised_matmul(dev, M, N, K):
+    got, want = _gemm_case(dev, M, N, K, seed=M + N + K)
+    cos = torch.nn.functional.cosine_similarity(got.flatten(), want.flatten(), dim=0).item()
+    assert cos >= 0.9995, cos
+    # fp32 accumulation of exact e4m3 products: only summation order differs, so far tighter than the cosine bar
+    err = (got - want).abs().max().item()
+    assert err <= 2e-2 * want.abs().max().item() + 1e-3, err
+
+
+@pytest.mark.parametrize("M", [1, 2, 8])
+def test_fp8_gemv_small_m(dev, M):
+    got, want = _gemm_case(dev, M, 515, 3072, seed=M)
+    assert (got - want).abs().max().item() <= 2e-2 * want.abs().max().item() + 1e-3
+
+
+def test_fp8_gemm_unit_scales_no_bias(dev):
+    """Reference mode (fp8_linear.py:41-48): scale_a = scale_b = 1, bare casts."""
+    got, want = _gemm_case(dev, 384, 512, 512, seed=5, bias=False, scaled=False)
+    assert (got - want).abs().max().item() <= 2e-2 * want.abs().max().item() + 1e-3
+
+
+def test_fp8_gemm_exact_on_small_integers(dev):
+    """Operands that are small integers make every partial sum exact: the result must be bit-identical."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    a = torch.randint(-3, 4, (512, 256), generator=g).float()
+    w = torch.randint(-2, 3, (320, 256), generator=g).float()
+    want = (a @ w.t()).bfloat16()
+    got = ops.fp8_gemm(a.to(torch.float8_e4m3fn).to(dev), w.to(torch.float8_e4m3fn).to(dev)).cpu()
+    assert torch.equal(got, want)
+
+
+def test_gemm_rejects_bad_arguments(dev):
+    from diffsynth_engine_amd import ops
+
+    a = torch.zeros(16, 24, dtype=torch.float8_e4m3fn, device=dev)
+    w = torch.zeros(16, 24, dtype=torch.float8_e4m3fn, device=dev)
+    with pytest.raises(ValueError):
+        ops.fp8_gemm(a, w)  # K % 16 != 0
+    with pytest.raises(ValueError):
+        ops.fp8_gemm(a.bfloat16(), w)
