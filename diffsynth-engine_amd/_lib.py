@@ -32,10 +32,10 @@ class AttnParams(ctypes.Structure):
         ("o", c_void_p * 2),
         ("sq", c_int64 * 2),
         ("skv", c_int64 * 2),
-        ("q_sb", c_int64), ("q_sh", c_int64), ("q_ss", c_int64),
-        ("k_sb", c_int64), ("k_sh", c_int64), ("k_ss", c_int64),
-        ("v_sb", c_int64), ("v_sh", c_int64), ("v_ss", c_int64),
-        ("o_sb", c_int64), ("o_sh", c_int64), ("o_ss", c_int64),
+        ("q_sb", c_int64 * 2), ("q_sh", c_int64 * 2), ("q_ss", c_int64 * 2),
+        ("k_sb", c_int64 * 2), ("k_sh", c_int64 * 2), ("k_ss", c_int64 * 2),
+        ("v_sb", c_int64 * 2), ("v_sh", c_int64 * 2), ("v_ss", c_int64 * 2),
+        ("o_sb", c_int64 * 2), ("o_sh", c_int64 * 2), ("o_ss", c_int64 * 2),
         ("batch", ctypes.c_int32), ("heads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
         ("softmax_scale", c_float),
         ("rope", c_void_p),
@@ -54,7 +54,7 @@ SIGNATURES = {
     "dsx_check_device": (c_int, []),
     "dsx_quant_fp8_rowwise": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p]),
     "dsx_absmax": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
-    "dsx_cast_fp8_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_void_p]),
+    "dsx_cast_fp8_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "dsx_fp8_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                              c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "dsx_attn_fwd": (c_int, [ctypes.POINTER(AttnParams), c_void_p]),

@@ -71,8 +71,8 @@ __device__ __forceinline__ u32x4 norm_rope_chunk(u32x4 raw, bool has_norm, float
       float x0 = v[2 * i], x1 = v[2 * i + 1];
       // same expression order as freqs[...,0]*x0 + freqs[...,1]*x1 with rows (c,-s) and (s,c)
       // (separately rounded products and sum, as separate torch ops produce them)
-      v[2 * i] = __fadd_rn(__fmul_rn(c, x0), __fmul_rn(-s, x1));
-      v[2 * i + 1] = __fadd_rn(__fmul_rn(s, x0), __fmul_rn(c, x1));
+      v[2 * i] = mul_add_unfused(c, x0, -s, x1);
+      v[2 * i + 1] = mul_add_unfused(s, x0, c, x1);
     }
   }
   u32x4 o;
@@ -105,12 +105,15 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
   const int64_t Skv = p.skv[0] + p.skv[1];
   const int64_t q0 = (int64_t)blockIdx.x * QB + wave * 64;
 
-  const uint16_t* qbase[2] = {(const uint16_t*)p.q[0], (const uint16_t*)p.q[1]};
-  const uint16_t* kbase[2] = {(const uint16_t*)p.k[0], (const uint16_t*)p.k[1]};
-  const uint16_t* vbase[2] = {(const uint16_t*)p.v[0], (const uint16_t*)p.v[1]};
-  const int64_t q_bh = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
-  const int64_t k_bh = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
-  const int64_t v_bh = (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+  const uint16_t* qbase[2];
+  const uint16_t* kbase[2];
+  const uint16_t* vbase[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    qbase[s] = (const uint16_t*)p.q[s] + (int64_t)b * p.q_sb[s] + (int64_t)h * p.q_sh[s];
+    kbase[s] = (const uint16_t*)p.k[s] + (int64_t)b * p.k_sb[s] + (int64_t)h * p.k_sh[s];
+    vbase[s] = (const uint16_t*)p.v[s] + (int64_t)b * p.v_sb[s] + (int64_t)h * p.v_sh[s];
+  }
   const float* rope = FUSED && p.rope ? p.rope + (int64_t)b * p.rope_sb : nullptr;
 
   // ---------------- Q fragments (B operand of S^T = K Q^T), loaded once ----------------
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
     int64_t row = q0 + qt * 32 + li;
     if (row >= Sq) row = Sq - 1;
     const int seg = row >= p.sq[0] ? 1 : 0;
-    const uint16_t* src = qbase[seg] + q_bh + (row - (seg ? p.sq[0] : 0)) * p.q_ss;
+    const uint16_t* src = qbase[seg] + (row - (seg ? p.sq[0] : 0)) * p.q_ss[seg];
     u32x4 raw[8];
 #pragma unroll
     for (int kc = 0; kc < 8; ++kc) raw[kc] = *reinterpret_cast<const u32x4*>(src + kc * 16 + g * 8);
@@ -165,7 +168,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
       if (key >= Skv) key = Skv - 1;
       const int seg = key >= p.skv[0] ? 1 : 0;
       const int64_t lrow = key - (seg ? p.skv[0] : 0);
-      u32x4 raw = *reinterpret_cast<const u32x4*>(kbase[seg] + k_bh + lrow * p.k_ss + ks_c * 8);
+      u32x4 raw = *reinterpret_cast<const u32x4*>(kbase[seg] + lrow * p.k_ss[seg] + ks_c * 8);
       if (FUSED) {
         const uint16_t* nw = (const uint16_t*)p.k_norm_w[seg];
         float rrms = 1.f;
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
       if (key >= Skv) key = Skv - 1;
       const int seg = key >= p.skv[0] ? 1 : 0;
       const int64_t lrow = key - (seg ? p.skv[0] : 0);
-      sv[i] = *reinterpret_cast<const u32x4*>(vbase[seg] + v_bh + lrow * p.v_ss + vs_dg * 8);
+      sv[i] = *reinterpret_cast<const u32x4*>(vbase[seg] + lrow * p.v_ss[seg] + vs_dg * 8);
     }
   };
   auto store_kv = [&](int buf) {
@@ -327,8 +330,10 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
   }
 
   // ---------------- normalise and store.  lane (g, j): query j, d = dt*32 + 8*(r/4) + 4g + r%4
-  uint16_t* obase[2] = {(uint16_t*)p.o[0], (uint16_t*)p.o[1]};
-  const int64_t o_bh = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+  uint16_t* obase[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+    obase[s] = (uint16_t*)p.o[s] + (int64_t)b * p.o_sb[s] + (int64_t)h * p.o_sh[s];
 #pragma unroll
   for (int qt = 0; qt < 2; ++qt) {
     const float l = halfwave_allsum(l_run[qt]);
@@ -336,7 +341,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
     const int64_t row = q0 + qt * 32 + li;
     if (row < Sq) {
       const int seg = row >= p.sq[0] ? 1 : 0;
-      uint16_t* dst = obase[seg] + o_bh + (row - (seg ? p.sq[0] : 0)) * p.o_ss;
+      uint16_t* dst = obase[seg] + (row - (seg ? p.sq[0] : 0)) * p.o_ss[seg];
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -398,12 +403,13 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
     return rc;
   const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
   if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 31) || Skv > (1ll << 31)) return DSX_EBADSHAPE;
-  const int64_t strides[12] = {p->q_sb, p->q_sh, p->q_ss, p->k_sb, p->k_sh, p->k_ss,
-                               p->v_sb, p->v_sh, p->v_ss, p->o_sb, p->o_sh, p->o_ss};
-  for (int i = 0; i < 12; ++i)
-    if (strides[i] & 7) return DSX_EALIGN;  // every row start must stay 16-byte aligned
-  if (p->q_ss < HD && Sq > 1) return DSX_EBADSHAPE;
-  if (p->o_ss < HD && Sq > 1) return DSX_EBADSHAPE;
+  for (int g = 0; g < 2; ++g) {
+    const int64_t strides[12] = {p->q_sb[g], p->q_sh[g], p->q_ss[g], p->k_sb[g], p->k_sh[g], p->k_ss[g],
+                                 p->v_sb[g], p->v_sh[g], p->v_ss[g], p->o_sb[g], p->o_sh[g], p->o_ss[g]};
+    for (int i = 0; i < 12; ++i)
+      if (strides[i] & 7) return DSX_EALIGN;  // every row start must stay 16-byte aligned
+    if (p->sq[g] > 1 && (p->o_ss[g] < HD || p->q_ss[g] < HD)) return DSX_EBADSHAPE;
+  }
   const bool fused = p->rope || p->q_norm_w[0] || p->q_norm_w[1] || p->k_norm_w[0] || p->k_norm_w[1];
   if (p->rope && (((uintptr_t)p->rope & 15) || (p->rope_sb & 3))) return DSX_EALIGN;
   if (p->rope && Sq != Skv) return DSX_EBADSHAPE;  // fused RoPE is defined for self/joint attention

@@ -91,14 +91,30 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-// tanh-GELU in fp32: 0.5*x*(1 + tanh(u)), u = sqrt(2/pi)*(x + 0.044715 x^3), evaluated as
-// x / (1 + exp(-2u)), which is the same function without the cancellation in 1 + tanh(u).
+// tanh-GELU in fp32 with the expression torch evaluates for approximate="tanh":
+// 0.5 * x * (1 + tanh(sqrt(2/pi) * (x + 0.044715 x^3))).  tanh(u) = 1 - 2/(exp(2u)+1) has an
+// absolute error of about one fp32 ulp of 1.0, like a library tanhf, and saturates to +-1 cleanly.
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
   const float kBeta = 0.7978845608028654f;  // sqrt(2/pi)
   const float kKappa = 0.044715f;
-  float u = kBeta * (x + kKappa * x * x * x);
-  float e = __builtin_amdgcn_exp2f(u * -2.8853900817779268f);  // exp(-2u)
-  return x / (1.0f + e);
+  const float u = kBeta * (x + kKappa * (x * x * x));
+  const float e = __builtin_amdgcn_exp2f(u * 2.8853900817779268f);  // exp(2u)
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  return 0.5f * x * (1.0f + t);
+}
+
+// Exactly rounded a*b + c*d with every operation rounded on its own (no FMA contraction), the
+// result separate torch kernels produce.
+__device__ __forceinline__ float mul_add_unfused(float a, float b, float c, float d) {
+#pragma clang fp contract(off)
+  const float p0 = a * b;
+  const float p1 = c * d;
+  return p0 + p1;
+}
+__device__ __forceinline__ float mul_then_add_unfused(float a, float b, float c) {
+#pragma clang fp contract(off)
+  const float p0 = a * b;
+  return p0 + c;
 }
 
 }  // namespace dsx

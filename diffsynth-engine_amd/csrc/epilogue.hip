@@ -36,10 +36,10 @@ __device__ __forceinline__ u32x4 pack8(const float* v) {
   o.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
   return o;
 }
-__device__ __forceinline__ u32x2 quant8(const float* v, float s) {
+__device__ __forceinline__ u32x2 quant8(const float* v, float inv) {
   uint32_t b[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) b[i] = f32_to_e4m3_bits(v[i] / s);
+  for (int i = 0; i < 8; ++i) b[i] = f32_to_e4m3_bits(v[i] * inv);
   u32x2 r;
   r.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
   r.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
@@ -69,12 +69,13 @@ __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint1
       }
     }
     amax = block_max(amax, red);
-    const float s = fmaxf(amax, 1e-12f) / 448.0f;
-    if (tid == 0) q_scale[row] = s;
+    amax = fmaxf(amax, 1e-12f);
+    const float inv = 448.0f / amax;
+    if (tid == 0) q_scale[row] = amax / 448.0f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = tid + i * 256;
-      if (c < nchunk) reinterpret_cast<u32x2*>(q)[c] = quant8(val[i], s);
+      if (c < nchunk) reinterpret_cast<u32x2*>(q)[c] = quant8(val[i], inv);
     }
   }
 }
@@ -220,13 +221,13 @@ __global__ __launch_bounds__(256) void euler_step_kernel(const void* __restrict_
     if (FP32) {
       const float a = reinterpret_cast<const float*>(lat)[i];
       const float b = reinterpret_cast<const float*>(v)[i];
-      reinterpret_cast<float*>(out)[i] = __fadd_rn(a, __fmul_rn(b, dt));
+      reinterpret_cast<float*>(out)[i] = mul_then_add_unfused(b, dt, a);
     } else {
       const float a = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(lat)[i]);
       const float b = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(v)[i]);
       // `model_outputs * dt` is a bf16 tensor, the sum is taken in fp32 and rounded once
-      const float prod = round_bf16(__fmul_rn(b, dt));
-      reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_bf16_bits(__fadd_rn(a, prod));
+      const float prod = round_bf16(b * dt);
+      reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)f32_to_bf16_bits(a + prod);
     }
   }
 }

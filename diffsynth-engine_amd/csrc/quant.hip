@@ -54,11 +54,11 @@ __global__ __launch_bounds__(256) void quant_rowwise_kernel(const uint16_t* __re
       if (SCALED) amax = fmaxf(amax, absmax_bf16x8(cache[i]));
     }
   }
-  float s = 1.0f;
+  float inv = 1.0f;
   if (SCALED) {
-    amax = wave_max(amax);
-    s = fmaxf(amax, 1e-12f) / 448.0f;
-    if (lane == 0) scale_out[row] = s;
+    amax = fmaxf(wave_max(amax), 1e-12f);
+    inv = 448.0f / amax;
+    if (lane == 0) scale_out[row] = amax / 448.0f;
   }
   u32x2* qr = reinterpret_cast<u32x2*>(q + row * ldq);
 #pragma unroll
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void quant_rowwise_kernel(const uint16_t* __re
       unpack_bf16x8(cache[i], v);
       if (SCALED) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = v[j] / s;
+        for (int j = 0; j < 8; ++j) v[j] = v[j] * inv;
       }
       qr[c] = pack_e4m3x8(v);
     }
@@ -93,15 +93,18 @@ __global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ x,
 
 template <bool FP32>
 __global__ __launch_bounds__(256) void cast_scaled_kernel(const void* __restrict__ x,
-                                                          const float* __restrict__ scale,
+                                                          const float* __restrict__ absmax,
+                                                          float* __restrict__ scale_out,
                                                           uint8_t* __restrict__ q, int64_t n) {
-  const bool scaled = scale != nullptr;
-  const float s = scaled ? *scale : 1.0f;
+  const bool scaled = absmax != nullptr;
+  const float amax = scaled ? fmaxf(*absmax, 1e-12f) : 1.0f;
+  const float inv = scaled ? 448.0f / amax : 1.0f;
+  if (scaled && blockIdx.x == 0 && threadIdx.x == 0) *scale_out = amax / 448.0f;
   int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     float v = FP32 ? reinterpret_cast<const float*>(x)[i]
                    : bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(x)[i]);
-    if (scaled) v = v / s;
+    if (scaled) v = v * inv;
     q[i] = (uint8_t)f32_to_e4m3_bits(v);
   }
 }
@@ -156,18 +159,20 @@ extern "C" int dsx_absmax(const void* x, int64_t n, int is_fp32, float* absmax_o
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
-extern "C" int dsx_cast_fp8_scaled(const void* x, int is_fp32, const float* scale, void* q,
-                                   int64_t n, void* stream) {
+extern "C" int dsx_cast_fp8_scaled(const void* x, int is_fp32, const float* absmax,
+                                   float* scale_out, void* q, int64_t n, void* stream) {
   using namespace dsx;
-  if (!x || !q) return DSX_ENULL;
+  if (!x || !q || (absmax && !scale_out)) return DSX_ENULL;
   if (n < 0) return DSX_EBADSHAPE;
   if (n == 0) return DSX_OK;
   hipStream_t st = (hipStream_t)stream;
   int64_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   if (is_fp32)
-    cast_scaled_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, scale, (uint8_t*)q, n);
+    cast_scaled_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, absmax, scale_out,
+                                                                           (uint8_t*)q, n);
   else
-    cast_scaled_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, scale, (uint8_t*)q, n);
+    cast_scaled_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(x, absmax, scale_out,
+                                                                            (uint8_t*)q, n);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }

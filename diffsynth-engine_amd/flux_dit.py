@@ -1,0 +1,205 @@
+"""Fused MI355X runner of the Flux DiT denoising step.
+
+Same inputs/outputs and state-dict names as ``FluxDiT.forward``
+(diffsynth_engine/models/flux/flux_dit.py:392-461), but the block bodies
+(FluxJointTransformerBlock.forward :219-236, FluxSingleTransformerBlock.forward :308-321,
+FluxJointAttention.forward :161-194) are issued as a fixed sequence of libdsx kernels:
+
+  AdaLN-modulate (+ e4m3 emission) -> FP8 GEMM -> flash attention reading q/k/v straight out of
+  the packed qkv projection by stride, RMSNorm + RoPE fused, text-first joint sequence from two base
+  pointers (no chunk/concat copies) -> quantise -> FP8 GEMM -> gated residual -> ...
+
+All Linear layers run as per-token x per-tensor scaled e4m3 GEMMs (``scaled=True``) or with the
+reference's bare casts and unit scales (``scaled=False``, utils/fp8_linear.py:28-60).
+"""
+import math
+from typing import Dict, Optional
+
+import torch
+
+from . import ops
+
+HIDDEN = 3072
+HEADS = 24
+HEAD_DIM = 128
+AXES_DIM = (16, 56, 56)
+THETA = 10000
+EPS = 1e-6
+
+
+class _Linear:
+    """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias."""
+
+    __slots__ = ("w", "s", "b", "n", "k")
+
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], scaled: bool):
+        if weight.dtype == ops.FP8:
+            self.w, self.s = weight, getattr(weight, "_dsx_scale", None)
+        else:
+            self.w, self.s = ops.quantize_weight_fp8(weight, scaled=scaled)
+        self.b = None if bias is None else bias.to(torch.bfloat16).contiguous()
+        self.n, self.k = self.w.shape
+
+    def __call__(self, a_q: torch.Tensor, a_s: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        return ops.fp8_gemm(a_q, self.w, a_s if self.s is not None else None, self.s, self.b, out=out)
+
+
+class FluxDiTRunner:
+    """Holds quantised weights of a Flux.1-dev-architecture DiT and runs one denoising step."""
+
+    def __init__(self, state_dict: Dict[str, torch.Tensor], num_double: int = 19, num_single: int = 38,
+                 scaled: bool = True, device="cuda:0"):
+        self.device = torch.device(device)
+        self.scaled = scaled
+        self.num_double, self.num_single = num_double, num_single
+        self.lin: Dict[str, _Linear] = {}
+        self.norm_w: Dict[str, torch.Tensor] = {}
+        # `state_dict` may be a mapping or any iterable of (name, tensor) pairs; the latter lets a caller
+        # stream a 12B-parameter model through without ever holding it unquantised
+        items = state_dict.items() if hasattr(state_dict, "items") else state_dict
+        for key, t in items:
+            if key.endswith(".weight") and t.dim() == 2:
+                self.lin[key[: -len(".weight")]] = _Linear(t.to(self.device), None, scaled)
+            elif key.endswith(".weight") and t.dim() == 1:
+                self.norm_w[key[: -len(".weight")]] = t.to(self.device, torch.bfloat16).contiguous()
+            elif key.endswith(".bias"):
+                self.lin[key[: -len(".bias")]].b = t.to(self.device, torch.bfloat16).contiguous()
+        self.has_guidance = "guidance_embedder.timestep_embedder.0" in self.lin
+        self._rope_cache = {}
+
+    # ------------------------------------------------------------------ small helpers
+    def _linear_bf16(self, x: torch.Tensor, name: str) -> torch.Tensor:
+        """quantise + GEMM for a bf16 activation (embedders and M=1 conditioning projections)."""
+        shp = x.shape
+        a_q, a_s = ops.quantize_fp8(x.reshape(-1, shp[-1]), scaled=self.scaled)
+        y = self.lin[name](a_q, a_s)
+        return y.view(*shp[:-1], y.shape[-1])
+
+    def _timestep_mlp(self, name: str, t: torch.Tensor) -> torch.Tensor:
+        """TimestepEmbeddings (models/basic/timestep.py:66-81): cos/sin features -> Linear -> SiLU -> Linear."""
+        half = 128
+        freq = torch.exp(-math.log(10000) * torch.arange(half, dtype=torch.float32, device=t.device) / half)
+        ang = t[:, None].float() * freq[None, :]
+        emb = torch.cat([torch.cos(ang), torch.sin(ang)], dim=-1).to(torch.bfloat16)
+        h = self._linear_bf16(emb, name + ".timestep_embedder.0")
+        return self._linear_bf16(torch.nn.functional.silu(h), name + ".timestep_embedder.2")
+
+    def _rope(self, text_ids: torch.Tensor, image_ids: torch.Tensor) -> torch.Tensor:
+        """(B,S,64,2) fp32 (cos, sin) table of RoPEEmbedding (transformer_helper.py:39-64), float64 angles."""
+        ids = torch.cat((text_ids, image_ids), dim=1).to(torch.float64)
+        cols = []
+        for a, dim in enumerate(AXES_DIM):
+            omega = 1.0 / (THETA ** (torch.arange(0, dim, 2, dtype=torch.float64, device=ids.device) / dim))
+            ang = ids[..., a].unsqueeze(-1) * omega
+            cols.append(torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1))
+        return torch.cat(cols, dim=-2).float().contiguous()
+
+    def _modulate_q(self, x, scale, shift):
+        """LayerNorm-modulate straight to the GEMM operand format."""
+        if self.scaled:
+            return ops.adaln_modulate(x, scale, shift, EPS, want_bf16=False, want_fp8=True)
+        return ops.quantize_fp8(ops.adaln_modulate(x, scale, shift, EPS), scaled=False)
+
+    def _gelu_q(self, h):
+        if self.scaled:
+            return ops.gelu_tanh(h, want_bf16=False, want_fp8=True)
+        return ops.quantize_fp8(ops.gelu_tanh(h), scaled=False)
+
+    # ------------------------------------------------------------------ blocks
+    def _joint_block(self, i: int, img, txt, mod_a, mod_b, rope):
+        """img (B,Si,d), txt (B,St,d); mod_*: (B, 6d) = shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp,
+        gate_mlp (transformer_helper.py:20)."""
+        pre = f"blocks.{i}."
+        B, Si, d = img.shape
+        St = txt.shape[1]
+        ma, mb = mod_a.chunk(6, dim=1), mod_b.chunk(6, dim=1)
+        L = self.lin
+        qa, sa = self._modulate_q(img, ma[1], ma[0])
+        qb, sb = self._modulate_q(txt, mb[1], mb[0])
+        qkv_a = L[pre + "attn.a_to_qkv"](qa.view(-1, d), sa).view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
+        qkv_b = L[pre + "attn.b_to_qkv"](qb.view(-1, d), sb).view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
+        o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
+        o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
+        nw = self.norm_w
+        ops.attention_bhsd(
+            qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:],
+            q2=qkv_a[:, :HEADS], k2=qkv_a[:, HEADS:2 * HEADS], v2=qkv_a[:, 2 * HEADS:],
+            rope=rope, q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
+            q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
+            out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2))
+        img = self._stream_tail(pre, "a", img, o_a.view(B * Si, d), ma)
+        txt = self._stream_tail(pre, "b", txt, o_b.view(B * St, d), mb)
+        return img, txt
+
+    def _stream_tail(self, pre, s, x, attn_out, m):
+        """out-projection, gated residual, LN-modulate, MLP, gated residual of one stream (flux_dit.py:226-234)."""
+        L = self.lin
+        B, S, d = x.shape
+        q, sc = ops.quantize_fp8(attn_out, scaled=self.scaled)
+        proj = L[pre + f"attn.{s}_to_out"](q, sc).view(B, S, d)
+        x = ops.gated_residual(x, proj, m[2])
+        q, sc = self._modulate_q(x, m[4], m[3])
+        h = L[pre + f"ff_{s}.0"](q.view(-1, d), sc)
+        q, sc = self._gelu_q(h)
+        h = L[pre + f"ff_{s}.2"](q, sc).view(B, S, d)
+        return ops.gated_residual(x, h, m[5])
+
+    def _single_block(self, i: int, x, mod, rope):
+        """x (B,S,d); mod (B,3d) = shift, scale, gate (transformer_helper.py:34)."""
+        pre = f"single_blocks.{i}."
+        B, S, d = x.shape
+        L = self.lin
+        shift, scale, gate = mod.chunk(3, dim=1)
+        q, sc = self._modulate_q(x, scale, shift)
+        h = L[pre + "to_qkv_mlp"](q.view(-1, d), sc)  # (B*S, 7d): [q | k | v | mlp]
+        cat = torch.empty((B * S, 5 * d), dtype=torch.bfloat16, device=x.device)
+        qkv = h.view(B, S, 7 * d)[:, :, : 3 * d].unflatten(2, (3 * HEADS, HEAD_DIM)).transpose(1, 2)
+        o = cat.view(B, S, 5 * d)[:, :, :d].unflatten(2, (HEADS, HEAD_DIM)).transpose(1, 2)
+        nw = self.norm_w
+        ops.attention_bhsd(qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:], rope=rope,
+                           q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"], eps=EPS, out=o)
+        ops.gelu_tanh(h[:, 3 * d:], want_bf16=True, out=cat[:, d:])
+        q, sc = ops.quantize_fp8(cat, scaled=self.scaled)
+        proj = L[pre + "proj_out"](q, sc).view(B, S, d)
+        return ops.gated_residual(x, proj, gate)
+
+    # ------------------------------------------------------------------ step
+    @torch.no_grad()
+    def forward(self, hidden_states, timestep, prompt_emb, pooled_prompt_emb, guidance, text_ids, image_ids=None):
+        dev = self.device
+        bf = torch.bfloat16
+        B, C, Hh, Ww = hidden_states.shape
+        if image_ids is None:
+            image_ids = torch.zeros(Hh // 2, Ww // 2, 3, device=dev)
+            image_ids[..., 1] += torch.arange(Hh // 2, device=dev)[:, None]
+            image_ids[..., 2] += torch.arange(Ww // 2, device=dev)[None, :]
+            image_ids = image_ids.reshape(1, -1, 3).repeat(B, 1, 1)
+        cond = self._timestep_mlp("time_embedder", timestep)
+        if self.has_guidance and guidance is not None:
+            cond = cond + self._timestep_mlp("guidance_embedder", guidance * 1000)
+        pooled = self._linear_bf16(pooled_prompt_emb.to(bf), "pooled_text_embedder.0")
+        cond = cond + self._linear_bf16(torch.nn.functional.silu(pooled), "pooled_text_embedder.2")
+        txt = self._linear_bf16(prompt_emb.to(bf), "context_embedder")
+        rope = self._rope(text_ids.to(dev), image_ids.to(dev))
+        x = hidden_states.to(bf).view(B, C, Hh // 2, 2, Ww // 2, 2).permute(0, 2, 4, 1, 3, 5)
+        img = self._linear_bf16(x.reshape(B, (Hh // 2) * (Ww // 2), C * 4), "x_embedder")
+
+        # every AdaLN projection consumes the same silu(cond): quantise it once
+        sc_q, sc_s = ops.quantize_fp8(torch.nn.functional.silu(cond), scaled=self.scaled)
+        for i in range(self.num_double):
+            mod_a = self.lin[f"blocks.{i}.norm1_a.linear"](sc_q, sc_s)
+            mod_b = self.lin[f"blocks.{i}.norm1_b.linear"](sc_q, sc_s)
+            img, txt = self._joint_block(i, img, txt, mod_a, mod_b, rope)
+        St = txt.shape[1]
+        x = torch.cat([txt, img], dim=1)
+        for i in range(self.num_single):
+            mod = self.lin[f"single_blocks.{i}.norm.linear"](sc_q, sc_s)
+            x = self._single_block(i, x, mod, rope)
+        x = x[:, St:]
+        mod = self.lin["final_norm_out.linear"](sc_q, sc_s)
+        scale, shift = mod.chunk(2, dim=1)  # AdaLayerNormContinuous: scale first (flux_dit.py:333)
+        q, s = self._modulate_q(x, scale, shift)
+        out = self.lin["final_proj_out"](q.view(-1, HIDDEN), s).view(B, Hh // 2, Ww // 2, C, 2, 2)
+        return out.permute(0, 3, 1, 4, 2, 5).reshape(B, C, Hh, Ww)
+
+    __call__ = forward

@@ -75,13 +75,13 @@ def quantize_weight_fp8(w: torch.Tensor, scaled: bool = True):
     w = w.contiguous()
     lib = _lib.load()
     is_fp32 = int(w.dtype == torch.float32)
-    scale = None
+    scale = amax = None
     if scaled:
         amax = torch.zeros((), dtype=torch.float32, device=w.device)
+        scale = torch.empty((), dtype=torch.float32, device=w.device)
         _lib.check(lib.dsx_absmax(_ptr(w), w.numel(), is_fp32, _ptr(amax), _stream()), "dsx_absmax")
-        scale = torch.clamp(amax, min=1e-12) / 448.0
     q = torch.empty(w.shape, dtype=FP8, device=w.device)
-    _lib.check(lib.dsx_cast_fp8_scaled(_ptr(w), is_fp32, _ptr(scale), _ptr(q), w.numel(), _stream()),
+    _lib.check(lib.dsx_cast_fp8_scaled(_ptr(w), is_fp32, _ptr(amax), _ptr(scale), _ptr(q), w.numel(), _stream()),
                "dsx_cast_fp8_scaled")
     return q, scale
 
@@ -158,21 +158,17 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     if q2 is not None and out2 is None:
         out2 = torch.empty((B, S2, H, D), dtype=_BF16, device=q.device).transpose(1, 2)
 
-    def same(a, b2, what):
-        if b2 is not None and _bhsd_strides(a) != _bhsd_strides(b2):
-            raise ValueError("both %s segments must share strides" % what)
-
-    same(q, q2, "q"); same(k, k2, "k"); same(v, v2, "v"); same(out, out2, "out")
     P.q[0], P.q[1] = _ptr(q), _ptr(q2)
     P.k[0], P.k[1] = _ptr(k), _ptr(k2)
     P.v[0], P.v[1] = _ptr(v), _ptr(v2)
     P.o[0], P.o[1] = _ptr(out), _ptr(out2)
     P.sq[0], P.sq[1] = S1, S2
     P.skv[0], P.skv[1] = Skv1, Skv2
-    P.q_sb, P.q_sh, P.q_ss = _bhsd_strides(q)
-    P.k_sb, P.k_sh, P.k_ss = _bhsd_strides(k)
-    P.v_sb, P.v_sh, P.v_ss = _bhsd_strides(v)
-    P.o_sb, P.o_sh, P.o_ss = _bhsd_strides(out)
+    for name, t1, t2 in (("q", q, q2), ("k", k, k2), ("v", v, v2), ("o", out, out2)):
+        for g, t in enumerate((t1, t2)):
+            if t is not None:
+                sb, sh, ss = _bhsd_strides(t)
+                getattr(P, name + "_sb")[g], getattr(P, name + "_sh")[g], getattr(P, name + "_ss")[g] = sb, sh, ss
     P.batch, P.heads, P.head_dim = B, H, D
     P.softmax_scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     keep = []

@@ -50,8 +50,9 @@ int dsx_check_device(void);
  *
  *   scale_out == NULL : bare cast, q[m,k] = e4m3_rne(x[m,k]); exactly torch's cast
  *                       (round-to-nearest-even, subnormals kept, |v| > 464 -> NaN).
- *   scale_out != NULL : dynamic per-token scale, s[m] = max(absmax(x[m,:]), 1e-12) / 448
- *                       (fp32 division), q[m,k] = e4m3_rne(float(x[m,k]) / s[m]).
+ *   scale_out != NULL : dynamic per-token scale, a = max(absmax(x[m,:]), 1e-12), s[m] = a / 448,
+ *                       q[m,k] = e4m3_rne(float(x[m,k]) * (448 / a)); both divisions and the
+ *                       product are single correctly rounded fp32 operations.
  * x: (M,K) bf16, row stride ldx; q: (M,K) e4m3, row stride ldq; K % 8 == 0.
  */
 int dsx_quant_fp8_rowwise(const void* x, int64_t ldx, void* q, int64_t ldq, float* scale_out,
@@ -65,11 +66,13 @@ int dsx_quant_fp8_rowwise(const void* x, int64_t ldx, void* q, int64_t ldq, floa
 int dsx_absmax(const void* x, int64_t n, int is_fp32, float* absmax_out, void* stream);
 
 /*
- * Per-tensor scaled cast: q[i] = e4m3_rne(float(x[i]) / *scale) (scale == NULL: bare cast).
+ * Per-tensor scaled cast.  absmax == NULL: bare cast q[i] = e4m3_rne(x[i]) (scale_out untouched).
+ * Otherwise a = max(*absmax, 1e-12), *scale_out = a / 448, q[i] = e4m3_rne(float(x[i]) * (448 / a));
+ * each division and the product is a single correctly rounded fp32 operation.
  * Replaces `module.weight.data.to(torch.float8_e4m3fn)` (fp8_linear.py:15).
  */
-int dsx_cast_fp8_scaled(const void* x, int is_fp32, const float* scale, void* q, int64_t n,
-                        void* stream);
+int dsx_cast_fp8_scaled(const void* x, int is_fp32, const float* absmax, float* scale_out, void* q,
+                        int64_t n, void* stream);
 
 /*
  * FP8 scaled GEMM with fused bias:
@@ -93,8 +96,8 @@ int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t ldw, const f
  * on q and k, and the text-first concat (flux_dit.py:176-178) through the two segments.
  *
  * The query sequence is the concatenation of up to two segments (segment 0 first), each read
- * from its own base pointer with shared strides; likewise keys/values and the output.
- * Element (b,h,s,d) of segment g of q lives at q[g][b*q_sb + h*q_sh + s*q_ss + d].
+ * from its own base pointer with its own strides; likewise keys/values and the output.
+ * Element (b,h,s,d) of segment g of q lives at q[g][b*q_sb[g] + h*q_sh[g] + s*q_ss[g] + d].
  */
 typedef struct dsx_attn_params {
   const void* q[2];   /* bf16; q[1] may be NULL when sq[1] == 0 */
@@ -103,10 +106,10 @@ typedef struct dsx_attn_params {
   void* o[2];         /* bf16 */
   int64_t sq[2];      /* query rows per segment  */
   int64_t skv[2];     /* key/value rows per segment */
-  int64_t q_sb, q_sh, q_ss;
-  int64_t k_sb, k_sh, k_ss;
-  int64_t v_sb, v_sh, v_ss;
-  int64_t o_sb, o_sh, o_ss;
+  int64_t q_sb[2], q_sh[2], q_ss[2];
+  int64_t k_sb[2], k_sh[2], k_ss[2];
+  int64_t v_sb[2], v_sh[2], v_ss[2];
+  int64_t o_sb[2], o_sh[2], o_ss[2];
   int32_t batch, heads, head_dim; /* head_dim must be 128 */
   float softmax_scale;            /* e.g. 1/sqrt(128) */
   /* Optional fused pre-processing of q and k (NULL = off):

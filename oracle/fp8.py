@@ -66,25 +66,27 @@ def cast_e4m3(x: torch.Tensor) -> torch.Tensor:
 
 
 def quantize_rowwise(x: torch.Tensor, scaled: bool = True):
-    """Per-token dynamic quantisation: s = max(absmax,1e-12)/448 (fp32), q = cast(float(x) / s).
+    """Per-token dynamic quantisation: a = max(absmax,1e-12), s = a/448, q = cast(float(x) * (448/a)), all fp32.
 
     ``scaled=False`` is the reference's bare cast with unit scale.
     """
     if not scaled:
         return cast_e4m3(x), None
     xf = x.float()
-    s = torch.clamp(xf.abs().amax(dim=-1), min=1e-12) / E4M3_MAX
-    q = (xf / s.unsqueeze(-1)).to(FP8)
-    return q, s
+    a = torch.clamp(xf.abs().amax(dim=-1), min=1e-12)
+    inv = torch.full_like(a, E4M3_MAX) / a  # a true fp32 division (``448.0 / a`` would be reciprocal * 448)
+    q = (xf * inv.unsqueeze(-1)).to(FP8)
+    return q, a / E4M3_MAX
 
 
 def quantize_weight(w: torch.Tensor, scaled: bool = True):
-    """fp8_linear.py:12-17 weight cast; scaled: per-tensor s_w = max(absmax,1e-12)/448."""
+    """fp8_linear.py:12-17 weight cast; scaled: a = max(absmax,1e-12), s_w = a/448, q = cast(w * (448/a))."""
     if not scaled:
         return cast_e4m3(w), None
     wf = w.float()
-    s = torch.clamp(wf.abs().amax(), min=1e-12) / E4M3_MAX
-    return (wf / s).to(FP8), s
+    a = torch.clamp(wf.abs().amax(), min=1e-12)
+    inv = torch.full_like(a, E4M3_MAX) / a
+    return (wf * inv).to(FP8), a / E4M3_MAX
 
 
 def scaled_linear(x_q, x_scale, w_q, w_scale, bias, out_dtype=torch.bfloat16):

@@ -44,7 +44,7 @@ def test_attn_params_struct_layout_matches_header():
 
     # 8 + 4 pointers/int64 pairs (12*8*... ) : q,k,v,o,sq,skv = 6*16; 12 strides*8; 3 int32 + float; rope, rope_sb;
     # 2*16 norm pointers; float + int32
-    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 8 + 16 + 8 + 8 + 32 + 8
+    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 32 + 8
 
 
 def test_null_and_shape_errors_without_touching_the_gpu():

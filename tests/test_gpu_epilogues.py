@@ -9,9 +9,11 @@ pytestmark = pytest.mark.gpu
 
 
 def _ulp_report(got, want):
-    """Fraction of elements that differ and max |diff| relative to max |want|."""
+    """Fraction of elements off by more than a bf16 ulp of |want| (or 1e-6 absolute, whichever is larger),
+    and max |diff| relative to max |want|."""
     d = (got.float() - want.float()).abs()
-    return (d > 0).float().mean().item(), (d.max() / want.float().abs().max()).item()
+    off = d > torch.maximum(want.float().abs() * 2 ** -7, torch.tensor(1e-6))
+    return off.float().mean().item(), (d.max() / want.float().abs().max()).item()
 
 
 @pytest.mark.parametrize("B,S,D", [(1, 40, 3072), (2, 17, 5120), (1, 5, 64), (1, 3, 16384)])
@@ -27,7 +29,7 @@ def test_adaln_modulate(dev, B, S, D):
     shd, scd = md.unsqueeze(1).chunk(6, dim=2)[:2]
     y, q, qs = ops.adaln_modulate(x.to(dev), scd, shd, want_bf16=True, want_fp8=True)
     frac, rel = _ulp_report(y.cpu(), want)
-    assert frac < 0.02 and rel <= 2 ** -6, (frac, rel)
+    assert frac < 1e-3 and rel <= 2 ** -6, (frac, rel)
     # the fused e4m3 emission must be the row quantiser applied to the kernel's own bf16 output
     wq, ws = ofp8.quantize_rowwise(y.cpu().reshape(-1, D), scaled=True)
     assert torch.equal(qs.cpu(), ws)
@@ -45,7 +47,7 @@ def test_adaln_affine_no_modulation(dev):
     want = O.layer_norm_modulate(x, None, None, 1e-6, w, b)
     got = ops.adaln_modulate(x.to(dev), None, None, ln_weight=w.to(dev), ln_bias=b.to(dev)).cpu()
     frac, rel = _ulp_report(got, want)
-    assert frac < 0.02 and rel <= 2 ** -6, (frac, rel)
+    assert frac < 1e-3 and rel <= 2 ** -6, (frac, rel)
 
 
 def test_layernorm_closed_form(dev):
@@ -83,7 +85,7 @@ def test_gelu_tanh(dev, rows, D):
     want = O.gelu_tanh(x)
     y, q, qs = ops.gelu_tanh(x.to(dev), want_bf16=True, want_fp8=True)
     frac, rel = _ulp_report(y.cpu(), want)
-    assert frac < 0.02 and rel <= 2 ** -7, (frac, rel)
+    assert frac < 1e-3 and rel <= 2 ** -7, (frac, rel)
     wq, ws = ofp8.quantize_rowwise(y.cpu(), scaled=True)
     assert torch.equal(qs.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8), wq.view(torch.uint8))
 
@@ -98,7 +100,7 @@ def test_gelu_all_bf16_inputs(dev):
     fin = torch.isfinite(want)
     assert torch.equal(torch.isnan(got), torch.isnan(want))
     d = (got[fin] - want[fin]).abs()
-    tol = want[fin].abs() * 2 ** -7 + 1e-30
+    tol = want[fin].abs() * 2 ** -7 + 1e-6
     assert bool((d <= tol).all())
 
 
@@ -110,7 +112,7 @@ def test_gelu_strided_slice_of_wider_buffer(dev):
     want = O.gelu_tanh(x[:, :, 9216:])
     got = ops.gelu_tanh(x.to(dev)[:, :, 9216:]).cpu()
     frac, rel = _ulp_report(got, want)
-    assert frac < 0.02 and rel <= 2 ** -7
+    assert frac < 1e-3 and rel <= 2 ** -7
 
 
 def test_flow_match_euler_step(dev):

@@ -1,0 +1,106 @@
+"""GPU parity of the fused Flux DiT runner against the oracle's restatement of FluxDiT.forward."""
+import pytest
+import torch
+
+from oracle import flux as oflux
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(side, n_txt, seed, device="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    lat = torch.randn(1, 16, side, side, generator=g).bfloat16()
+    prompt = torch.randn(1, n_txt, 4096, generator=g).bfloat16()
+    pooled = torch.randn(1, 768, generator=g).bfloat16()
+    return dict(hidden_states=lat.to(device), timestep=torch.tensor([500.0], device=device),
+                prompt_emb=prompt.to(device), pooled_prompt_emb=pooled.to(device),
+                guidance=torch.tensor([3.5], device=device), text_ids=torch.zeros(1, n_txt, 3, device=device))
+
+
+def _cos(a, b):
+    return torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item()
+
+
+def _floor(o_cpu, o_dev):
+    """FP8 rounding makes the step chaotic: a 1-ulp bf16 difference in one row's absmax re-grids the whole
+    row.  The same oracle code run by two torch backends (CPU vs device) therefore agrees only to a cosine
+    that depends on depth; the runner is required to be as close to the oracle as the oracle is to itself
+    (minus a small margin), and to reach 0.999 outright wherever the oracle does."""
+    return min(0.999, _cos(o_cpu, o_dev) - 0.002)
+
+
+@pytest.mark.parametrize("mode,scaled", [("fp8_scaled", True), ("fp8_ref", False)])
+def test_two_block_step_matches_cpu_oracle(dev, mode, scaled):
+    """1 double + 1 single block, 16x16 latent (64 image tokens) + 24 text tokens, oracle on the CPU in bf16."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=3, bias_std=0.02)
+    inp = _inputs(16, 24, seed=4)
+    want = oflux.flux_dit_forward(oflux.Params(sd, mode), **inp, num_double=1, num_single=1)
+    sd_dev = {k: v.to(dev) for k, v in sd.items()}
+    inp_dev = {k: v.to(dev) for k, v in inp.items()}
+    want_dev = oflux.flux_dit_forward(oflux.Params(sd_dev, mode), **inp_dev, num_double=1, num_single=1).cpu()
+    got = FluxDiTRunner(sd, 1, 1, scaled=scaled, device=dev)(**inp_dev).cpu()
+    assert got.shape == want.shape
+    assert _cos(got, want) >= 0.995
+    assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
+
+
+def test_deeper_step_matches_oracle(dev):
+    """4 double + 6 single blocks at 32x32 latent (256 image + 64 text tokens), oracle on the CPU."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(4, 6, dtype=torch.bfloat16, seed=5, bias_std=0.02)
+    inp = _inputs(32, 64, seed=6)
+    want = oflux.flux_dit_forward(oflux.Params(sd, "fp8_scaled"), **inp, num_double=4, num_single=6)
+    sd_dev = {k: v.to(dev) for k, v in sd.items()}
+    inp_dev = {k: v.to(dev) for k, v in inp.items()}
+    want_dev = oflux.flux_dit_forward(oflux.Params(sd_dev, "fp8_scaled"), **inp_dev, num_double=4, num_single=6).cpu()
+    got = FluxDiTRunner(sd_dev, 4, 6, scaled=True, device=dev)(**inp_dev).cpu()
+    assert _cos(got, want) >= 0.99
+    assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
+
+
+def test_blocks_teacher_forced_against_oracle(dev):
+    """Each block fed the oracle's own inputs (no error carried between blocks): joint block and single block
+    outputs against the CPU oracle.  One block holds 4-5 chained e4m3 quantisations, hence 0.9995 rather than 1."""
+    from diffsynth_engine_amd import ops
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+    from oracle import dit_ops as O
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=9, bias_std=0.02)
+    P = oflux.Params(sd, "fp8_scaled")
+    R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    g = torch.Generator().manual_seed(10)
+    St, side = 40, 12
+    img = torch.randn(1, side * side, 3072, generator=g).bfloat16()
+    txt = torch.randn(1, St, 3072, generator=g).bfloat16()
+    cond = torch.randn(1, 3072, generator=g).bfloat16()
+    ids = torch.cat([torch.zeros(1, St, 3), oflux.image_ids(2 * side, 2 * side, 1, "cpu", torch.float32)], dim=1)
+    freqs = O.rope_table(ids, oflux.AXES_DIM, oflux.THETA)
+    rope = ops.rope_table_from_freqs(freqs).to(dev)
+    want_a, want_b = oflux.joint_block(P, 0, img, txt, cond, freqs)
+    sc_q, sc_s = ops.quantize_fp8(torch.nn.functional.silu(cond).to(dev), scaled=True)
+    mod_a = R.lin["blocks.0.norm1_a.linear"](sc_q, sc_s)
+    mod_b = R.lin["blocks.0.norm1_b.linear"](sc_q, sc_s)
+    got_a, got_b = R._joint_block(0, img.to(dev), txt.to(dev), mod_a, mod_b, rope)
+    assert _cos(got_a, want_a) >= 0.9995 and _cos(got_b, want_b) >= 0.9995, (_cos(got_a, want_a), _cos(got_b, want_b))
+    x = torch.cat([txt, img], dim=1)
+    want = oflux.single_block(P, 0, x, cond, freqs)
+    got = R._single_block(0, x.to(dev), R.lin["single_blocks.0.norm.linear"](sc_q, sc_s), rope)
+    assert _cos(got, want) >= 0.9995, _cos(got, want)
+
+
+def test_zero_gates_make_blocks_identity(dev):
+    """With every AdaLN projection zeroed, gates are 0 and the residual stream must pass through unchanged,
+    so the output depends only on the embedders and the final layer: equal for 0+0 and 2+2 blocks."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(2, 2, dtype=torch.bfloat16, seed=7)
+    for k in sd:
+        if ".norm1_a.linear." in k or ".norm1_b.linear." in k or ".norm.linear." in k:
+            sd[k] = torch.zeros_like(sd[k])
+    inp = {k: v.to(dev) for k, v in _inputs(16, 8, seed=8).items()}
+    a = FluxDiTRunner(sd, 2, 2, device=dev)(**inp).cpu()
+    b = FluxDiTRunner(sd, 0, 0, device=dev)(**inp).cpu()
+    assert torch.equal(a, b)
