@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the DiT denoising-step hot path on one MI355X.
+
+Headline workload: one full Flux.1-dev-architecture DiT denoising step (19 double-stream + 38
+single-stream blocks, hidden 3072, 24 heads x 128, 1024x1024 image = 4096 image tokens + 512 text
+tokens, batch 1), random-init weights N(0, 0.02) quantised to e4m3 with per-tensor scales, activations
+quantised per token, synthetic N(0,1) inputs.  A "step" is one FluxDiTRunner.forward.
+
+Prints ONE JSON line.  `roofline` describes the dominant kernel (the FP8 GEMM, ~80 % of the step's
+flops): algorithmic flops 2*M*N*K of every large GEMM launched in the timed region divided by the sum of
+their durations, measured with events on the launch stream.  `cpu_baseline` times the CPU oracle
+(pure-torch restatement of the reference path) on the host cores for a bounded sample.
+Secondary figures (attention kernel TFLOP/s at S=4608, per-shape GEMM TFLOP/s, HBM GB/s of the
+bandwidth-bound kernels) ride along under "detail".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8 = 5.0e15   # MI355X dense fp8 MFMA, flop/s
+PEAK_BF16 = 2.5e15  # MI355X dense bf16 MFMA, flop/s
+PEAK_HBM = 8.0e12   # bytes/s
+
+HIDDEN, HEADS, HEAD_DIM = 3072, 24, 128
+N_IMG, N_TXT = 4096, 512
+
+
+def flux_state_dict_stream(num_double, num_single, device, seed=0, std=0.02):
+    """Yield (name, tensor) pairs of a random Flux.1-dev-architecture DiT, generated on the device one tensor
+    at a time (weights N(0,std) bf16, biases 0, RMSNorm weights 1) so that the runner can quantise as it goes."""
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    d = HIDDEN
+
+    def lin(name, n_in, n_out):
+        yield name + ".weight", (torch.randn(n_out, n_in, generator=g, device=device) * std).to(torch.bfloat16)
+        yield name + ".bias", torch.zeros(n_out, dtype=torch.bfloat16, device=device)
+
+    def ones(name):
+        yield name + ".weight", torch.ones(HEAD_DIM, dtype=torch.bfloat16, device=device)
+
+    yield from lin("time_embedder.timestep_embedder.0", 256, d)
+    yield from lin("time_embedder.timestep_embedder.2", d, d)
+    yield from lin("guidance_embedder.timestep_embedder.0", 256, d)
+    yield from lin("guidance_embedder.timestep_embedder.2", d, d)
+    yield from lin("pooled_text_embedder.0", 768, d)
+    yield from lin("pooled_text_embedder.2", d, d)
+    yield from lin("context_embedder", 4096, d)
+    yield from lin("x_embedder", 64, d)
+    for i in range(num_double):
+        p = f"blocks.{i}."
+        yield from lin(p + "norm1_a.linear", d, 6 * d)
+        yield from lin(p + "norm1_b.linear", d, 6 * d)
+        yield from lin(p + "attn.a_to_qkv", d, 3 * d)
+        yield from lin(p + "attn.b_to_qkv", d, 3 * d)
+        for n in ("norm_q_a", "norm_k_a", "norm_q_b", "norm_k_b"):
+            yield from ones(p + "attn." + n)
+        yield from lin(p + "attn.a_to_out", d, d)
+        yield from lin(p + "attn.b_to_out", d, d)
+        yield from lin(p + "ff_a.0", d, 4 * d)
+        yield from lin(p + "ff_a.2", 4 * d, d)
+        yield from lin(p + "ff_b.0", d, 4 * d)
+        yield from lin(p + "ff_b.2", 4 * d, d)
+    for i in range(num_single):
+        p = f"single_blocks.{i}."
+        yield from lin(p + "norm.linear", d, 3 * d)
+        yield from lin(p + "to_qkv_mlp", d, 7 * d)
+        yield from ones(p + "norm_q_a")
+        yield from ones(p + "norm_k_a")
+        yield from lin(p + "proj_out", 5 * d, d)
+    yield from lin("final_norm_out.linear", d, 2 * d)
+    yield from lin("final_proj_out", d, 64)
+
+
+def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
+    """Algorithmic flops of one step: 2MNK of every Linear with M > 1 plus 4*S^2*D*H per attention."""
+    d, S = HIDDEN, n_img + n_txt
+    per_tok_double = 2 * d * (3 * d + d + 4 * d + 4 * d)
+    gemm = num_double * S * per_tok_double + num_single * S * 2 * d * (7 * d + 5 * d)
+    gemm += n_txt * 2 * 4096 * d + n_img * 2 * 64 * d + n_img * 2 * d * 64
+    attn = (num_double + num_single) * 4 * S * S * HEAD_DIM * HEADS
+    return gemm, attn
+
+
+class GemmTimer:
+    """Brackets every fp8_gemm launch with events on the launch stream (torch's current stream, which is the
+    stream handed to the C-ABI) and accumulates algorithmic flops for launches with M > 8."""
+
+    def __init__(self, torch, ops):
+        self.torch, self.ops = torch, ops
+        self.records = []
+        self._orig = ops.fp8_gemm
+
+    def __enter__(self):
+        torch, orig, rec = self.torch, self._orig, self.records
+
+        def timed(a_q, w_q, *args, **kw):
+            M, K = a_q.shape
+            if M <= 8:
+                return orig(a_q, w_q, *args, **kw)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = orig(a_q, w_q, *args, **kw)
+            e1.record()
+            rec.append((e0, e1, 2.0 * M * K * w_q.shape[0]))
+            return out
+
+        self.ops.fp8_gemm = timed
+        return self
+
+    def __exit__(self, *exc):
+        self.ops.fp8_gemm = self._orig
+
+    def summary(self):
+        self.torch.cuda.synchronize()
+        secs = sum(e0.elapsed_time(e1) for e0, e1, _ in self.records) * 1e-3
+        flops = sum(f for _, _, f in self.records)
+        return len(self.records), flops, secs
+
+
+def time_kernel(torch, fn, iters=30, warmup=5):
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / iters
+
+
+def micro_benchmarks(torch, ops, dev):
+    """Per-kernel figures at the sizes of the Flux-1024 step: configs[1] GEMM shapes, configs[2] attention,
+    and the bandwidth-bound kernels."""
+    detail = {}
+    g = torch.Generator(device=dev).manual_seed(0)
+    M = N_IMG + N_TXT
+    gem = {}
+    for K, N in ((3072, 9216), (3072, 3072), (3072, 12288), (12288, 3072), (3072, 21504), (15360, 3072)):
+        x = torch.randn(M, K, generator=g, device=dev, dtype=torch.bfloat16)
+        x[:, torch.randperm(K, generator=g, device=dev)[: max(1, -(-K // 1000))]] *= 20
+        w = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+        bias = torch.randn(N, generator=g, device=dev).to(torch.bfloat16)
+        wq, ws = ops.quantize_weight_fp8(w)
+        xq, xs = ops.quantize_fp8(x)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+        t = time_kernel(torch, lambda: ops.fp8_gemm(xq, wq, xs, ws, bias, out=out))
+        tq = time_kernel(torch, lambda: ops.quantize_fp8(x))
+        fl = 2.0 * M * N * K
+        gem[f"{K}x{N}"] = {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
+                           "frac_fp8_peak": round(fl / t / PEAK_FP8, 4),
+                           "quant_us": round(tq * 1e6, 1), "quant_gbps": round((M * K * 3 + 4 * M) / tq / 1e9, 1)}
+        del x, w, wq, xq, out
+    detail["fp8_gemm_M4608"] = gem
+
+    S = M
+    q = torch.randn(1, HEADS, S, HEAD_DIM, generator=g, device=dev, dtype=torch.bfloat16)
+    k = torch.randn(1, HEADS, S, HEAD_DIM, generator=g, device=dev, dtype=torch.bfloat16)
+    v = torch.randn(1, HEADS, S, HEAD_DIM, generator=g, device=dev, dtype=torch.bfloat16)
+    out = torch.empty(1, S, HEADS, HEAD_DIM, dtype=torch.bfloat16, device=dev).transpose(1, 2)
+    fl = 4.0 * S * S * HEAD_DIM * HEADS
+    t = time_kernel(torch, lambda: ops.attention_bhsd(q, k, v, out=out))
+    att = {"plain": {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1), "frac_bf16_peak": round(fl / t / PEAK_BF16, 4)}}
+    # fused RMSNorm + 3-axis RoPE (16,56,56), ids: 512 text rows at 0, then (0,r,c) over 64x64
+    ids = torch.zeros(1, S, 3, dtype=torch.float64, device=dev)
+    rc = torch.arange(64, device=dev, dtype=torch.float64)
+    ids[0, N_TXT:, 1] = rc.repeat_interleave(64)
+    ids[0, N_TXT:, 2] = rc.repeat(64)
+    cols = []
+    for a, dim in enumerate((16, 56, 56)):
+        omega = 1.0 / (10000 ** (torch.arange(0, dim, 2, dtype=torch.float64, device=dev) / dim))
+        ang = ids[..., a].unsqueeze(-1) * omega
+        cols.append(torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1))
+    rope = torch.cat(cols, dim=-2).float().contiguous()
+    w1 = torch.ones(HEAD_DIM, dtype=torch.bfloat16, device=dev)
+    t = time_kernel(torch, lambda: ops.attention_bhsd(q, k, v, out=out, rope=rope, q_norm_w=w1, k_norm_w=w1))
+    att["fused_rmsnorm_rope"] = {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
+                                 "frac_bf16_peak": round(fl / t / PEAK_BF16, 4)}
+    detail["attention_S4608_H24_D128"] = att
+
+    x = torch.randn(1, S, HIDDEN, generator=g, device=dev, dtype=torch.bfloat16)
+    y = torch.randn(1, S, HIDDEN, generator=g, device=dev, dtype=torch.bfloat16)
+    mod = torch.randn(1, 3 * HIDDEN, generator=g, device=dev, dtype=torch.bfloat16)
+    sh, sc, gt = mod.chunk(3, dim=1)
+    h = torch.randn(S, 4 * HIDDEN, generator=g, device=dev, dtype=torch.bfloat16)
+    t1 = time_kernel(torch, lambda: ops.adaln_modulate(x, sc, sh, want_bf16=True))
+    t1q = time_kernel(torch, lambda: ops.adaln_modulate(x, sc, sh, want_bf16=False, want_fp8=True))
+    t2 = time_kernel(torch, lambda: ops.gated_residual(x, y, gt))
+    t3 = time_kernel(torch, lambda: ops.gelu_tanh(h))
+    t3q = time_kernel(torch, lambda: ops.gelu_tanh(h, want_bf16=False, want_fp8=True))
+    n = S * HIDDEN
+    detail["epilogues"] = {
+        "adaln_modulate_bf16": {"us": round(t1 * 1e6, 1), "gbps": round(4 * n / t1 / 1e9, 1)},
+        "adaln_modulate_fp8": {"us": round(t1q * 1e6, 1), "gbps": round(3 * n / t1q / 1e9, 1)},
+        "gated_residual": {"us": round(t2 * 1e6, 1), "gbps": round(6 * n / t2 / 1e9, 1)},
+        "gelu_tanh_bf16": {"us": round(t3 * 1e6, 1), "gbps": round(16 * n / t3 / 1e9, 1)},
+        "gelu_tanh_fp8": {"us": round(t3q * 1e6, 1), "gbps": round(12 * n / t3q / 1e9, 1)},
+    }
+    return detail
+
+
+def cpu_baseline(num_double, num_single):
+    """The oracle (fp32, torch SDPA-equivalent eager attention) on the host cores: ONE double-stream and ONE
+    single-stream block at the full 4096+512 tokens, extrapolated to 19 + 38 blocks."""
+    import torch
+
+    from oracle import dit_ops as O
+    from oracle import flux as oflux
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    sd = oflux.init_params(1, 1, dtype=torch.float32, seed=0)
+    P = oflux.Params(sd, "plain")
+    g = torch.Generator().manual_seed(0)
+    img = torch.randn(1, N_IMG, HIDDEN, generator=g)
+    txt = torch.randn(1, N_TXT, HIDDEN, generator=g)
+    cond = torch.randn(1, HIDDEN, generator=g)
+    ids = torch.cat([torch.zeros(1, N_TXT, 3), oflux.image_ids(128, 128, 1, "cpu", torch.float32)], dim=1)
+    freqs = O.rope_table(ids, oflux.AXES_DIM, oflux.THETA)
+    sdpa = torch.nn.functional.scaled_dot_product_attention
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        a, b = oflux.joint_block(P, 0, img, txt, cond, freqs, attn=sdpa)
+        t1 = time.perf_counter()
+        oflux.single_block(P, 0, torch.cat([b, a], dim=1), cond, freqs, attn=sdpa)
+        t2 = time.perf_counter()
+    ms = ((t1 - t0) * num_double + (t2 - t1) * num_single) * 1e3
+    return {"value": round(ms, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "oracle fp32 on host: 1 double block (%.2f s) + 1 single block (%.2f s) at 4096+512 tokens, "
+                      "extrapolated x%d + x%d (embedders and final layer excluded)" % (t1 - t0, t2 - t1, num_double, num_single)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--double", type=int, default=19)
+    ap.add_argument("--single", type=int, default=38)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-micro", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X; this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+
+    from diffsynth_engine_amd import _lib, ops
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X (no GPU visible)")
+    rc = _lib.load().dsx_check_device()
+    if rc:
+        sys.exit("bench.py: " + _lib.strerror(rc))
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    runner = FluxDiTRunner(flux_state_dict_stream(args.double, args.single, dev), args.double, args.single,
+                           scaled=True, device=dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    inp = dict(
+        hidden_states=torch.randn(1, 16, 128, 128, generator=g, device=dev).to(torch.bfloat16),
+        timestep=torch.tensor([500.0], device=dev),
+        prompt_emb=torch.randn(1, N_TXT, 4096, generator=g, device=dev).to(torch.bfloat16),
+        pooled_prompt_emb=torch.randn(1, 768, generator=g, device=dev).to(torch.bfloat16),
+        guidance=torch.tensor([3.5], device=dev),
+        text_ids=torch.zeros(1, N_TXT, 3, device=dev),
+    )
+    for _ in range(args.warmup):
+        out = runner(**inp)
+    torch.cuda.synchronize()
+    with GemmTimer(torch, ops) as gt:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = runner(**inp)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        n_gemm, gemm_flops, gemm_secs = gt.summary()
+    assert torch.isfinite(out.float()).all().item(), "non-finite output"
+    ms = (t1 - t0) * 1e3 / args.steps
+
+    gemm_fl, attn_fl = step_flops(args.double, args.single)
+    t_ideal = gemm_fl / PEAK_FP8 + attn_fl / PEAK_BF16
+    achieved = gemm_flops / gemm_secs if gemm_secs > 0 else 0.0
+    result = {
+        "metric": "flux_1024x1024_fp8_dit_step_ms",
+        "value": round(ms, 3),
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 3),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3 GEMM (fp32 accumulate) + bf16 attention",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[3]: full Flux.1-dev-architecture DiT, one denoising step, "
+                               "%d double + %d single blocks, 4096 image + 512 text tokens, batch 1, "
+                               "random init N(0,0.02), e4m3 weights (per-tensor scale), per-token activation scale"
+                               % (args.double, args.single)},
+        "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 1), "peak": PEAK_FP8 / 1e12,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8, 4), "traffic": None,
+                     "kernel": "fp8_gemm_kernel", "launches": n_gemm,
+                     "avg_launch_us": round(gemm_secs / max(n_gemm, 1) * 1e6, 1)},
+        "step_roofline": {"algorithmic_tflop": round((gemm_fl + attn_fl) / 1e12, 2),
+                          "ideal_ms": round(t_ideal * 1e3, 2), "frac": round(t_ideal * 1e3 / ms, 4)},
+    }
+    if not args.no_micro:
+        result["detail"] = micro_benchmarks(torch, ops, dev)
+    del runner
+    torch.cuda.empty_cache()
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args.double, args.single)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
