@@ -1,21 +1,27 @@
 // FP8 e4m3 scaled GEMM for gfx950:  out = bf16((A * W^T) * a_scale[m] * w_scale + bias[n]).
 //
-// Both operands are K-contiguous ("TN"), which is what v_mfma_f32_32x32x64_f8f6f4 wants: lane
-// (g = lane/32, i = lane%32) feeds 32 consecutive K bytes of row i for the A operand and of
-// column i for the B operand.  Any permutation of K that is applied to both operands leaves
-// the product unchanged, so the tile loader only has to keep the two consistent.
+// Both operands are K-contiguous, which is what v_mfma_f32_32x32x64_f8f6f4 wants: lane
+// (g = lane/32, i = lane%32) feeds 32 K-bytes of row i of the first operand and of column i of
+// the second.  Any permutation of K applied to both operands leaves the product unchanged, so
+// the loaders only have to keep the two consistent.
 //
-// Tiling: 256x256 output tile per workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
-// tiles (256 fp32 accumulator registers), K step 128 bytes, two LDS stages (2 x 64 KiB).
-// LDS rows are 128 B (8 chunks of 16 B); chunk c of row r is stored at chunk c ^ ((r/2)&7) so
-// that 16 lanes reading 16 consecutive rows at the same logical chunk hit 16 distinct
-// 16-byte bank groups.
+// The kernels compute C^T tiles (first operand = W rows, second = A rows): the accumulator of
+// lane (g, j) then holds ONE token m = j and four consecutive output features per register
+// quad, so the per-token scale is a per-lane constant and the bf16 results leave as 8-byte stores.
+//
+// Main kernel: 256x256 output tile per workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
+// tiles (256 fp32 accumulators), K step 128 bytes, two LDS stages of 64 KiB filled by
+// global_load_lds_dwordx4 (HBM/L2 -> LDS without staging registers) one full K step ahead,
+// MFMA operand fragments double-buffered in registers so that LDS reads overlap the MFMAs.
+// LDS rows are 128 B (8 chunks of 16 B); chunk c of row r lives at chunk c ^ ((r/2)&7), which
+// makes 16 lanes reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
 #include "common.h"
 
 namespace dsx {
 
 constexpr int BM = 256, BN = 256, BK = 128;
-constexpr int kStageBytes = (BM + BN) * BK;  // 64 KiB
+constexpr int kTileBytes = 256 * BK;           // one operand tile, 32 KiB
+constexpr int kStageBytes = 2 * kTileBytes;    // W tile + A tile, 64 KiB
 
 __device__ __forceinline__ int lds_off(int row, int chunk) {
   return row * BK + ((chunk ^ ((row >> 1) & 7)) << 4);
@@ -51,6 +57,54 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
   tn = rem / gsz;
 }
 
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// Store one C^T accumulator tile set of a wave.  acc[tn][tm]: rows n, columns m (see header).
+__device__ __forceinline__ void store_ct(const GemmArgs& p, f32x16 (&acc)[4][4], int n_base,
+                                         int m_base, int g, int li) {
+  const float ws = p.w_scale ? *p.w_scale : 1.0f;
+  const bool vec_ok = ((p.ldo & 3) == 0) && ((p.N & 3) == 0) && (((uintptr_t)p.out & 7) == 0);
+#pragma unroll
+  for (int tm = 0; tm < 4; ++tm) {
+    const int m = m_base + tm * 32 + li;
+    if (m >= p.M) continue;
+    const float sc = (p.a_scale ? p.a_scale[m] : 1.0f) * ws;
+    uint16_t* orow = p.out + (int64_t)m * p.ldo;
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int n = n_base + tn * 32 + 8 * rq + 4 * g;
+        if (vec_ok) {
+          if (n < p.N) {
+            float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+            if (p.bias) {
+              const u32x2 bw = *reinterpret_cast<const u32x2*>(p.bias + n);
+              b0 = bf16_lo(bw.x); b1 = bf16_hi(bw.x); b2 = bf16_lo(bw.y); b3 = bf16_hi(bw.y);
+            }
+            u32x2 o;
+            o.x = pack_bf16x2(acc[tn][tm][4 * rq + 0] * sc + b0, acc[tn][tm][4 * rq + 1] * sc + b1);
+            o.y = pack_bf16x2(acc[tn][tm][4 * rq + 2] * sc + b2, acc[tn][tm][4 * rq + 3] * sc + b3);
+            *reinterpret_cast<u32x2*>(orow + n) = o;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e < p.N) {
+              const float bj = p.bias ? bf16_bits_to_f32(p.bias[n + e]) : 0.f;
+              orow[n + e] = (uint16_t)f32_to_bf16_bits(acc[tn][tm][4 * rq + e] * sc + bj);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Main kernel: K % 128 == 0.
+// ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int tm, tn;
@@ -61,44 +115,46 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wn = wave >> 1, wm = wave & 1;
   const int g = lane >> 5, li = lane & 31;
   const int m0 = tm * BM, n0 = tn * BN;
-  const int kchunks = p.K >> 4;  // 16-byte chunks per row
 
-  // --- global -> register staging: thread handles chunks id = tid + 256*i, i < 8, per operand
-  const int st_c = tid & 7;        // chunk within the 128-byte K slab
-  const int st_r = tid >> 3;       // row 0..31 (+32*i)
-  const uint8_t* a_src[8];
+  // ---- async tile loads: every wave instruction fills 1 KiB of LDS = 8 rows x 128 B; lane l
+  //      lands at row l/8, physical chunk l%8, so it must fetch logical chunk (l%8) ^ swz(row).
+  const int ld_r = lane >> 3, ld_p = lane & 7;
   const uint8_t* w_src[8];
+  const uint8_t* a_src[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    int ra = min(m0 + st_r + 32 * i, p.M - 1);
-    int rw = min(n0 + st_r + 32 * i, p.N - 1);
-    a_src[i] = p.a + (int64_t)ra * p.lda + st_c * 16;
-    w_src[i] = p.w + (int64_t)rw * p.ldw + st_c * 16;
+    const int row = (wave * 8 + i) * 8 + ld_r;
+    const int c = ld_p ^ ((row >> 1) & 7);
+    w_src[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.ldw + c * 16;
+    a_src[i] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.lda + c * 16;
   }
-  int st_off[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) st_off[i] = lds_off(st_r + 32 * i, st_c);
-
-  u32x4 sa[8], sw[8];
-  auto load_stage = [&](int kt) {
-    const bool in = (kt * 8 + st_c) < kchunks;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      sa[i] = in ? *reinterpret_cast<const u32x4*>(a_src[i] + (int64_t)kt * BK) : u32x4{0, 0, 0, 0};
-      sw[i] = in ? *reinterpret_cast<const u32x4*>(w_src[i] + (int64_t)kt * BK) : u32x4{0, 0, 0, 0};
-    }
+  // one of the 16 async 1-KiB loads of a K step (8 for W, 8 for A)
+  auto issue_load = [&](int kt, int buf, int idx) {
+    uint8_t* dst = smem + buf * kStageBytes + (idx & 1) * kTileBytes + (wave * 8 + (idx >> 1)) * 1024;
+    const uint8_t* src = ((idx & 1) ? a_src[idx >> 1] : w_src[idx >> 1]) + (int64_t)kt * BK;
+    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
   };
-  auto store_stage = [&](int buf) {
-    uint8_t* sA = smem + buf * kStageBytes;
-    uint8_t* sB = sA + BM * BK;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      *reinterpret_cast<u32x4*>(sA + st_off[i]) = sa[i];
-      *reinterpret_cast<u32x4*>(sB + st_off[i]) = sw[i];
-    }
+
+  // ---- fragment reads: fragment set = 4 W tiles + 4 A tiles, each tile two 16-byte halves
+  const int w_row = wn * 128 + li;
+  const int a_row = wm * 128 + li;
+  struct Frags {
+    i32x4 w[4][2];
+    i32x4 a[4][2];
+  };
+  // read #idx (0..15) of the fragment set of K sub-step ks from stage `buf`
+  auto read_frag = [&](Frags& f, int buf, int ks, int idx) {
+    const uint8_t* sW = smem + buf * kStageBytes;
+    const uint8_t* sA = sW + kTileBytes;
+    const int t = idx >> 2, half = idx & 1, is_a = (idx >> 1) & 1;
+    const int c = ks * 4 + g * 2 + half;
+    if (is_a)
+      f.a[t][half] = *reinterpret_cast<const i32x4*>(sA + lds_off(a_row + t * 32, c));
+    else
+      f.w[t][half] = *reinterpret_cast<const i32x4*>(sW + lds_off(w_row + t * 32, c));
   };
 
   f32x16 acc[4][4];
@@ -109,66 +165,126 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int nk = (p.K + BK - 1) / BK;
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
+  auto mfma_one = [&](const Frags& f, int idx) {
+    const int i = idx >> 2, j = idx & 3;
+    const i32x8 fw = {f.w[i][0].x, f.w[i][0].y, f.w[i][0].z, f.w[i][0].w,
+                      f.w[i][1].x, f.w[i][1].y, f.w[i][1].z, f.w[i][1].w};
+    const i32x8 fa = {f.a[j][0].x, f.a[j][0].y, f.a[j][0].z, f.a[j][0].w,
+                      f.a[j][1].x, f.a[j][1].y, f.a[j][1].z, f.a[j][1].w};
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fw, fa, acc[i][j], 0, 0, 0, 0, 0, 0);
+  };
 
-  // per-lane LDS row bases of the fragments this wave reads
-  const int a_row = wm * 128 + li;
-  const int b_row = wn * 128 + li;
+  // Schedule of one K step (tile kt in stage kt&1):
+  //   half A: 16 MFMAs on F0 (K bytes 0..63), each followed by one LDS read of F1 (bytes 64..127)
+  //   barrier: tile kt+1 (requested one full step earlier) has landed; stage kt&1 is free again
+  //   half B: 16 MFMAs on F1; the first four are each followed by four async loads of tile kt+2
+  //           into stage kt&1, all sixteen by one LDS read of the next F0 (tile kt+1, bytes 0..63)
+  // sched_barrier(0) pins that interleaving, so LDS and HBM latency sit under MFMA issue.
+  const int nk = p.K / BK;
+  Frags f0, f1;
+#pragma unroll
+  for (int idx = 0; idx < 16; ++idx) issue_load(0, 0, idx);
+  __syncthreads();  // includes vmcnt(0): tile 0 is in LDS
+#pragma unroll
+  for (int idx = 0; idx < 16; ++idx) read_frag(f0, 0, 0, idx);
+#pragma unroll
+  for (int idx = 0; idx < 16; ++idx) issue_load(min(1, nk - 1), 1, idx);
 
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
-    if (kt + 1 < nk) load_stage(kt + 1);
-    const uint8_t* sA = smem + buf * kStageBytes;
-    const uint8_t* sB = sA + BM * BK;
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+      mfma_one(f0, idx);
+      read_frag(f1, buf, 1, idx);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+    // Past the last tile the loads re-fetch tile nk-1 into a stage nobody reads again and the
+    // LDS reads return values nobody uses: cheaper than branches inside the pinned schedule.
+    const int kt2 = min(kt + 2, nk - 1);
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+      mfma_one(f1, idx);
+      if (idx < 4) {
+#pragma unroll
+        for (int l = 0; l < 4; ++l) issue_load(kt2, buf, idx * 4 + l);
+      }
+      read_frag(f0, buf ^ 1, 0, idx);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is released
+
+  store_ct(p, acc, n0 + wn * 128, m0 + wm * 128, g, li);
+}
+
+// ------------------------------------------------------------------------------------------
+// Generic kernel for K % 128 != 0 (K % 16 == 0): register-staged loads with a zero-filled K tail.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fp8_gemm_ragged_k_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int tm, tn;
+  bool valid;
+  tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn, valid);
+  if (!valid) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wn = wave >> 1, wm = wave & 1;
+  const int g = lane >> 5, li = lane & 31;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int kchunks = p.K >> 4;
+  const int st_c = tid & 7, st_r = tid >> 3;
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  uint8_t* sW = smem;
+  uint8_t* sA = smem + kTileBytes;
+  const int nk = (p.K + BK - 1) / BK;
+  for (int kt = 0; kt < nk; ++kt) {
+    const bool in = (kt * 8 + st_c) < kchunks;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = st_r + 32 * i;
+      u32x4 wv = {0, 0, 0, 0}, av = {0, 0, 0, 0};
+      if (in) {
+        wv = *reinterpret_cast<const u32x4*>(p.w + (int64_t)min(n0 + row, p.N - 1) * p.ldw +
+                                             (int64_t)kt * BK + st_c * 16);
+        av = *reinterpret_cast<const u32x4*>(p.a + (int64_t)min(m0 + row, p.M - 1) * p.lda +
+                                             (int64_t)kt * BK + st_c * 16);
+      }
+      *reinterpret_cast<u32x4*>(sW + lds_off(row, st_c)) = wv;
+      *reinterpret_cast<u32x4*>(sA + lds_off(row, st_c)) = av;
+    }
+    __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      i32x8 fa[4], fb[4];
+      i32x8 fw[4], fa[4];
       const int c0 = ks * 4 + g * 2;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int ra = a_row + t * 32, rb = b_row + t * 32;
-        i32x4 a_lo = *reinterpret_cast<const i32x4*>(sA + lds_off(ra, c0));
-        i32x4 a_hi = *reinterpret_cast<const i32x4*>(sA + lds_off(ra, c0 + 1));
-        i32x4 b_lo = *reinterpret_cast<const i32x4*>(sB + lds_off(rb, c0));
-        i32x4 b_hi = *reinterpret_cast<const i32x4*>(sB + lds_off(rb, c0 + 1));
+        const int rw = wn * 128 + t * 32 + li, ra = wm * 128 + t * 32 + li;
+        const i32x4 w_lo = *reinterpret_cast<const i32x4*>(sW + lds_off(rw, c0));
+        const i32x4 w_hi = *reinterpret_cast<const i32x4*>(sW + lds_off(rw, c0 + 1));
+        const i32x4 a_lo = *reinterpret_cast<const i32x4*>(sA + lds_off(ra, c0));
+        const i32x4 a_hi = *reinterpret_cast<const i32x4*>(sA + lds_off(ra, c0 + 1));
+        fw[t] = i32x8{w_lo.x, w_lo.y, w_lo.z, w_lo.w, w_hi.x, w_hi.y, w_hi.z, w_hi.w};
         fa[t] = i32x8{a_lo.x, a_lo.y, a_lo.z, a_lo.w, a_hi.x, a_hi.y, a_hi.z, a_hi.w};
-        fb[t] = i32x8{b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w};
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0,
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fw[i], fa[j], acc[i][j], 0, 0,
                                                                       0, 0, 0, 0);
     }
-    if (kt + 1 < nk) store_stage(buf ^ 1);
     __syncthreads();
   }
-
-  // --- epilogue.  C layout of a 32x32 tile: lane (g, li) register r holds
-  //     row 8*(r/4) + 4*g + (r%4), column li.
-  const float ws = p.w_scale ? *p.w_scale : 1.0f;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int col = n0 + wn * 128 + j * 32 + li;
-    const bool col_ok = col < p.N;
-    const float bj = (p.bias && col_ok) ? bf16_bits_to_f32(p.bias[col]) : 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-        if (col_ok && row < p.M) {
-          const float as = p.a_scale ? p.a_scale[row] : 1.0f;
-          float v = acc[i][j][r] * (as * ws) + bj;
-          p.out[(int64_t)row * p.ldo + col] = (uint16_t)f32_to_bf16_bits(v);
-        }
-      }
-    }
-  }
+  store_ct(p, acc, n0 + wn * 128, m0 + wm * 128, g, li);
 }
 
 // Small-M path (M <= 8): one wave per output column, fp32 FMA over dequantised bytes.
@@ -220,7 +336,8 @@ extern "C" int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t l
   if (!a || !w || !out) return DSX_ENULL;
   if (M < 0 || N <= 0 || K <= 0 || (K & 15) || lda < K || ldw < K || ldo < N) return DSX_EBADSHAPE;
   if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return DSX_EBADSHAPE;
-  if ((lda & 15) || (ldw & 15) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)out & 1))
+  if ((lda & 15) || (ldw & 15) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)out & 1) ||
+      ((uintptr_t)bias & 1))
     return DSX_EALIGN;
   if (M == 0) return DSX_OK;
   GemmArgs p;
@@ -249,10 +366,15 @@ extern "C" int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t l
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)fp8_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            2 * kStageBytes) != hipSuccess)
+                            2 * kStageBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
       return DSX_ELAUNCH;
     attr_set = true;
   }
-  fp8_gemm_kernel<<<dim3((unsigned)grid), dim3(256), 2 * kStageBytes, st>>>(p);
+  if ((K % BK) == 0)
+    fp8_gemm_kernel<<<dim3((unsigned)grid), dim3(256), 2 * kStageBytes, st>>>(p);
+  else
+    fp8_gemm_ragged_k_kernel<<<dim3((unsigned)grid), dim3(256), kStageBytes, st>>>(p);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }

@@ -18,7 +18,7 @@ def _inputs(side, n_txt, seed, device="cpu"):
 
 
 def _cos(a, b):
-    return torch.nn.functional.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item()
+    return torch.nn.functional.cosine_similarity(a.float().flatten().cpu(), b.float().flatten().cpu(), dim=0).item()
 
 
 def _floor(o_cpu, o_dev):
