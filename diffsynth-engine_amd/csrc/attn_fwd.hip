@@ -355,11 +355,12 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(dsx_attn_params p) {
   }
 }
 
-// Standalone RMSNorm + RoPE: one wave per (b,h,s) row... 16 lanes per row, 4 rows per wave.
+// Standalone RMSNorm + RoPE: 16 lanes per (b,h,s) row, 16 rows per workgroup.  `out` may alias `x`
+// (in-place): every thread reads its 16 bytes before it writes them.
 __global__ __launch_bounds__(256) void rmsnorm_rope_kernel(
-    const uint16_t* __restrict__ x, int64_t x_sb, int64_t x_sh, int64_t x_ss,
+    const uint16_t* x, int64_t x_sb, int64_t x_sh, int64_t x_ss,
     const uint16_t* __restrict__ norm_w, float eps, const float* __restrict__ rope, int64_t rope_sb,
-    int64_t rope_pos0, uint16_t* __restrict__ out, int64_t o_sb, int64_t o_sh, int64_t o_ss,
+    int64_t rope_pos0, uint16_t* out, int64_t o_sb, int64_t o_sh, int64_t o_ss,
     int heads, int64_t seq) {
   const int c = threadIdx.x & 15;
   const int64_t s = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);

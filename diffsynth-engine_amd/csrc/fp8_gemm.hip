@@ -102,9 +102,89 @@ __device__ __forceinline__ void store_ct(const GemmArgs& p, f32x16 (&acc)[4][4],
   }
 }
 
+// LDS-staged store of a wave's 128 (m) x 128 (n) block: the C^T accumulators are scaled, biased,
+// rounded to bf16 and written to a wave-private LDS region as [m][n] rows (272-byte pitch: 256 data
+// bytes + 16 pad, so 8-byte column writes of 32 consecutive rows spread over the banks), then read
+// back as 16-byte chunks along n so that 16 lanes emit one contiguous 256-byte row segment.
+constexpr int kEpiPitch = 272;
+constexpr int kEpiBytesPerWave = 128 * kEpiPitch;  // 34 816
+constexpr int kMainLdsBytes = 160 * 1024;  // five operand stages; the epilogue staging (136 KiB) reuses them
+
+// Per-lane epilogue operands, fetched in one batch so that their latency is paid once.
+struct EpiOperands {
+  u32x2 bias[4][4];  // [tn][rq]: 4 consecutive bf16 at n = tn*32 + 8*rq + 4*g
+  float sc[4];       // [tm]: a_scale[m] * w_scale
+};
+__device__ __forceinline__ void load_epi_operands(const GemmArgs& p, EpiOperands& e, int n_base,
+                                                  int m_base, int lane) {
+  const int g = lane >> 5, li = lane & 31;
+  const float ws = p.w_scale ? *p.w_scale : 1.0f;
+#pragma unroll
+  for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      const int n = n_base + tn * 32 + 8 * rq + 4 * g;
+      e.bias[tn][rq] = (p.bias && n < p.N) ? *reinterpret_cast<const u32x2*>(p.bias + n) : u32x2{0, 0};
+    }
+#pragma unroll
+  for (int tm = 0; tm < 4; ++tm) {
+    const int m = m_base + tm * 32 + li;
+    e.sc[tm] = (p.a_scale && m < p.M ? p.a_scale[m] : 1.0f) * ws;
+  }
+}
+
+__device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][4], const EpiOperands& e,
+                                             uint8_t* wave_lds, int n_base, int m_base, int lane) {
+  const int g = lane >> 5, li = lane & 31;
+#pragma unroll
+  for (int tm = 0; tm < 4; ++tm) {
+    const float sc = e.sc[tm];
+    uint8_t* lrow = wave_lds + (tm * 32 + li) * kEpiPitch;
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int nl = tn * 32 + 8 * rq + 4 * g;
+        const u32x2 bw = e.bias[tn][rq];
+        u32x2 o;
+        o.x = pack_bf16x2(acc[tn][tm][4 * rq + 0] * sc + bf16_lo(bw.x),
+                          acc[tn][tm][4 * rq + 1] * sc + bf16_hi(bw.x));
+        o.y = pack_bf16x2(acc[tn][tm][4 * rq + 2] * sc + bf16_lo(bw.y),
+                          acc[tn][tm][4 * rq + 3] * sc + bf16_hi(bw.y));
+        *reinterpret_cast<u32x2*>(lrow + nl * 2) = o;
+      }
+    }
+  }
+  // the region is private to this wave: its own LDS writes only have to have completed
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  __builtin_amdgcn_wave_barrier();
+  const int ch = lane & 15, r0 = lane >> 4;
+  const int n = n_base + ch * 8;
+#pragma unroll
+  for (int it = 0; it < 32; ++it) {
+    const int ml = it * 4 + r0;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
+    if (m_base + ml < p.M && n < p.N)
+      *reinterpret_cast<u32x4*>(p.out + (int64_t)(m_base + ml) * p.ldo + n) = v;
+  }
+}
+
 // ------------------------------------------------------------------------------------------
-// Main kernel: K % 128 == 0.
+// Main kernel: K % 128 == 0.  Five LDS stages of one 64-byte K slab each (W tile 256x64 + A tile
+// 256x64 = 32 KiB per stage, 160 KiB in all), filled by global_load_lds_dwordx4 four slabs ahead:
+// a slab needs ~0.5 us just to stream through the CU's vector memory path on top of the L2/HBM
+// latency, so a one-slab lead leaves the MFMAs waiting on memory.
 // ------------------------------------------------------------------------------------------
+constexpr int SK = 64;                        // K bytes per stage
+constexpr int NSTAGE = 5;
+constexpr int kSlabTile = 256 * SK;           // one operand, 16 KiB
+constexpr int kSlabBytes = 2 * kSlabTile;     // 32 KiB
+
+// 64-byte rows: 16-byte chunk c of row r lives at chunk c ^ ((r/4)&3); four rows span the 64 banks.
+__device__ __forceinline__ int slab_off(int row, int chunk) {
+  return row * SK + ((chunk ^ ((row >> 2) & 3)) << 4);
+}
+
 __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int tm, tn;
@@ -119,42 +199,48 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   const int g = lane >> 5, li = lane & 31;
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // ---- async tile loads: every wave instruction fills 1 KiB of LDS = 8 rows x 128 B; lane l
-  //      lands at row l/8, physical chunk l%8, so it must fetch logical chunk (l%8) ^ swz(row).
-  const int ld_r = lane >> 3, ld_p = lane & 7;
-  const uint8_t* w_src[8];
-  const uint8_t* a_src[8];
+  // ---- async loads: one wave instruction fills 1 KiB of LDS = 16 rows x 64 B; lane l lands at
+  //      row l/4, physical chunk l%4, so it fetches logical chunk (l%4) ^ swz(row).
+  //      Per slab a wave issues 8 instructions: 4 for its 64 W rows, 4 for its 64 A rows.
+  const int ld_r = lane >> 2, ld_p = lane & 3;
+  const uint8_t* w_src[4];
+  const uint8_t* a_src[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = (wave * 8 + i) * 8 + ld_r;
-    const int c = ld_p ^ ((row >> 1) & 7);
+  for (int i = 0; i < 4; ++i) {
+    const int row = (wave * 4 + i) * 16 + ld_r;
+    const int c = ld_p ^ ((row >> 2) & 3);
+#ifdef DSX_EXPERIMENT_SAMETILE
+    w_src[i] = p.w + (int64_t)min(row, p.N - 1) * p.ldw + c * 16;
+    a_src[i] = p.a + (int64_t)min(row, p.M - 1) * p.lda + c * 16;
+#else
     w_src[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.ldw + c * 16;
     a_src[i] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.lda + c * 16;
+#endif
   }
-  // one of the 16 async 1-KiB loads of a K step (8 for W, 8 for A)
-  auto issue_load = [&](int kt, int buf, int idx) {
-    uint8_t* dst = smem + buf * kStageBytes + (idx & 1) * kTileBytes + (wave * 8 + (idx >> 1)) * 1024;
-    const uint8_t* src = ((idx & 1) ? a_src[idx >> 1] : w_src[idx >> 1]) + (int64_t)kt * BK;
+  const int nk = p.K / SK;
+  auto issue_load = [&](int kt, int stage, int idx) {
+    kt = min(kt, nk - 1);  // past the end: re-fetch the last slab into a stage nobody reads again
+    uint8_t* dst = smem + stage * kSlabBytes + (idx & 1) * kSlabTile + (wave * 4 + (idx >> 1)) * 1024;
+    const uint8_t* src = ((idx & 1) ? a_src[idx >> 1] : w_src[idx >> 1]) + (int64_t)kt * SK;
     __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
   };
 
-  // ---- fragment reads: fragment set = 4 W tiles + 4 A tiles, each tile two 16-byte halves
+  // ---- fragments: 4 W tiles + 4 A tiles, two 16-byte halves each = 16 LDS reads per slab
   const int w_row = wn * 128 + li;
   const int a_row = wm * 128 + li;
   struct Frags {
     i32x4 w[4][2];
     i32x4 a[4][2];
   };
-  // read #idx (0..15) of the fragment set of K sub-step ks from stage `buf`
-  auto read_frag = [&](Frags& f, int buf, int ks, int idx) {
-    const uint8_t* sW = smem + buf * kStageBytes;
-    const uint8_t* sA = sW + kTileBytes;
+  auto read_frag = [&](Frags& f, int stage, int idx) {
+    const uint8_t* sW = smem + stage * kSlabBytes;
+    const uint8_t* sA = sW + kSlabTile;
     const int t = idx >> 2, half = idx & 1, is_a = (idx >> 1) & 1;
-    const int c = ks * 4 + g * 2 + half;
+    const int c = g * 2 + half;
     if (is_a)
-      f.a[t][half] = *reinterpret_cast<const i32x4*>(sA + lds_off(a_row + t * 32, c));
+      f.a[t][half] = *reinterpret_cast<const i32x4*>(sA + slab_off(a_row + t * 32, c));
     else
-      f.w[t][half] = *reinterpret_cast<const i32x4*>(sW + lds_off(w_row + t * 32, c));
+      f.w[t][half] = *reinterpret_cast<const i32x4*>(sW + slab_off(w_row + t * 32, c));
   };
 
   f32x16 acc[4][4];
@@ -174,48 +260,49 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fw, fa, acc[i][j], 0, 0, 0, 0, 0, 0);
   };
 
-  // Schedule of one K step (tile kt in stage kt&1):
-  //   half A: 16 MFMAs on F0 (K bytes 0..63), each followed by one LDS read of F1 (bytes 64..127)
-  //   barrier: tile kt+1 (requested one full step earlier) has landed; stage kt&1 is free again
-  //   half B: 16 MFMAs on F1; the first four are each followed by four async loads of tile kt+2
-  //           into stage kt&1, all sixteen by one LDS read of the next F0 (tile kt+1, bytes 0..63)
-  // sched_barrier(0) pins that interleaving, so LDS and HBM latency sit under MFMA issue.
-  const int nk = p.K / BK;
+  // One step: slab s is in registers (fc).  Behind the barrier slab s+1 is in LDS (only the 16
+  // newest async loads, slabs s+2 and s+3, may still be in flight) and stage (s+4)%5 = (s-1)%5 has
+  // been read for the last time by every wave.  16 MFMAs, each followed by one LDS read of slab
+  // s+1 and, for the first eight, one async load of slab s+4; sched_barrier pins that order.
+  auto step = [&](int s, const Frags& fc, Frags& fn) {
+    __builtin_amdgcn_s_waitcnt(0x4070);  // vmcnt(16) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    const int st_next = (s + 1) % NSTAGE, st_load = (s + 4) % NSTAGE;
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+      mfma_one(fc, idx);
+      read_frag(fn, st_next, idx);
+      if (idx < 8) issue_load(s + 4, st_load, idx);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
   Frags f0, f1;
 #pragma unroll
-  for (int idx = 0; idx < 16; ++idx) issue_load(0, 0, idx);
-  __syncthreads();  // includes vmcnt(0): tile 0 is in LDS
+  for (int s = 0; s < 4; ++s)
 #pragma unroll
-  for (int idx = 0; idx < 16; ++idx) read_frag(f0, 0, 0, idx);
+    for (int idx = 0; idx < 8; ++idx) issue_load(s, s, idx);
+  __builtin_amdgcn_s_waitcnt(0x4f78);  // vmcnt(24): slab 0 has landed
+  __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int idx = 0; idx < 16; ++idx) issue_load(min(1, nk - 1), 1, idx);
+  for (int idx = 0; idx < 16; ++idx) read_frag(f0, 0, idx);
 
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-#pragma unroll
-    for (int idx = 0; idx < 16; ++idx) {
-      mfma_one(f0, idx);
-      read_frag(f1, buf, 1, idx);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    __syncthreads();
-    // Past the last tile the loads re-fetch tile nk-1 into a stage nobody reads again and the
-    // LDS reads return values nobody uses: cheaper than branches inside the pinned schedule.
-    const int kt2 = min(kt + 2, nk - 1);
-#pragma unroll
-    for (int idx = 0; idx < 16; ++idx) {
-      mfma_one(f1, idx);
-      if (idx < 4) {
-#pragma unroll
-        for (int l = 0; l < 4; ++l) issue_load(kt2, buf, idx * 4 + l);
-      }
-      read_frag(f0, buf ^ 1, 0, idx);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+  for (int s = 0; s < nk; s += 2) {  // nk is even (K % 128 == 0)
+    step(s, f0, f1);
+    step(s + 1, f1, f0);
   }
-  __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is released
+  __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is reused
 
-  store_ct(p, acc, n0 + wn * 128, m0 + wm * 128, g, li);
+  const bool vec_ok = ((p.ldo & 7) == 0) && ((p.N & 7) == 0) && (((uintptr_t)p.out & 15) == 0) &&
+                      (!p.bias || ((uintptr_t)p.bias & 7) == 0);
+  if (vec_ok) {
+    EpiOperands epi;
+    load_epi_operands(p, epi, n0 + wn * 128, m0 + wm * 128, lane);
+    __syncthreads();  // every wave is done reading the operand stages
+    store_ct_lds(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 128, lane);
+  } else {
+    store_ct(p, acc, n0 + wn * 128, m0 + wm * 128, g, li);
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -366,14 +453,14 @@ extern "C" int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t l
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)fp8_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            2 * kStageBytes) != hipSuccess ||
+                            kMainLdsBytes) != hipSuccess ||
         hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
       return DSX_ELAUNCH;
     attr_set = true;
   }
-  if ((K % BK) == 0)
-    fp8_gemm_kernel<<<dim3((unsigned)grid), dim3(256), 2 * kStageBytes, st>>>(p);
+  if ((K % 128) == 0)
+    fp8_gemm_kernel<<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(p);
   else
     fp8_gemm_ragged_k_kernel<<<dim3((unsigned)grid), dim3(256), kStageBytes, st>>>(p);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;

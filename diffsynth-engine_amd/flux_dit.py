@@ -48,9 +48,11 @@ class FluxDiTRunner:
     """Holds quantised weights of a Flux.1-dev-architecture DiT and runs one denoising step."""
 
     def __init__(self, state_dict: Dict[str, torch.Tensor], num_double: int = 19, num_single: int = 38,
-                 scaled: bool = True, device="cuda:0"):
+                 scaled: bool = True, device="cuda:0", fuse_rope_in_attention: bool = False):
         self.device = torch.device(device)
         self.scaled = scaled
+        # True: RMSNorm/RoPE applied inside the attention kernel's tile loads; False: one in-place pre-pass
+        self.fuse_rope_in_attention = fuse_rope_in_attention
         self.num_double, self.num_single = num_double, num_single
         self.lin: Dict[str, _Linear] = {}
         self.norm_w: Dict[str, torch.Tensor] = {}
@@ -121,12 +123,22 @@ class FluxDiTRunner:
         o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         nw = self.norm_w
-        ops.attention_bhsd(
-            qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:],
-            q2=qkv_a[:, :HEADS], k2=qkv_a[:, HEADS:2 * HEADS], v2=qkv_a[:, 2 * HEADS:],
-            rope=rope, q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
-            q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
-            out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2))
+        qb_, kb_, vb_ = qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:]
+        qa_, ka_, va_ = qkv_a[:, :HEADS], qkv_a[:, HEADS:2 * HEADS], qkv_a[:, 2 * HEADS:]
+        if self.fuse_rope_in_attention:
+            ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, rope=rope,
+                               q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
+                               q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
+                               out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2))
+        else:
+            # RMSNorm + RoPE rewrite q and k in place inside the packed projections (one read + one write of
+            # q and k) so that the attention kernel streams K without re-normalising it once per query tile
+            ops.rmsnorm_rope(qb_, nw[pre + "attn.norm_q_b"], rope, 0, EPS, out=qb_)
+            ops.rmsnorm_rope(kb_, nw[pre + "attn.norm_k_b"], rope, 0, EPS, out=kb_)
+            ops.rmsnorm_rope(qa_, nw[pre + "attn.norm_q_a"], rope, St, EPS, out=qa_)
+            ops.rmsnorm_rope(ka_, nw[pre + "attn.norm_k_a"], rope, St, EPS, out=ka_)
+            ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2),
+                               out2=o_a.transpose(1, 2))
         img = self._stream_tail(pre, "a", img, o_a.view(B * Si, d), ma)
         txt = self._stream_tail(pre, "b", txt, o_b.view(B * St, d), mb)
         return img, txt
@@ -156,8 +168,14 @@ class FluxDiTRunner:
         qkv = h.view(B, S, 7 * d)[:, :, : 3 * d].unflatten(2, (3 * HEADS, HEAD_DIM)).transpose(1, 2)
         o = cat.view(B, S, 5 * d)[:, :, :d].unflatten(2, (HEADS, HEAD_DIM)).transpose(1, 2)
         nw = self.norm_w
-        ops.attention_bhsd(qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:], rope=rope,
-                           q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"], eps=EPS, out=o)
+        q_, k_, v_ = qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:]
+        if self.fuse_rope_in_attention:
+            ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
+                               eps=EPS, out=o)
+        else:
+            ops.rmsnorm_rope(q_, nw[pre + "norm_q_a"], rope, 0, EPS, out=q_)
+            ops.rmsnorm_rope(k_, nw[pre + "norm_k_a"], rope, 0, EPS, out=k_)
+            ops.attention_bhsd(q_, k_, v_, out=o)
         ops.gelu_tanh(h[:, 3 * d:], want_bf16=True, out=cat[:, d:])
         q, sc = ops.quantize_fp8(cat, scaled=self.scaled)
         proj = L[pre + "proj_out"](q, sc).view(B, S, d)

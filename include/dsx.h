@@ -129,7 +129,8 @@ int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
 
 /*
  * Standalone RMSNorm + RoPE of q and k (same arithmetic and rounding points as the fused
- * option of dsx_attn_fwd), written to a dense (B,H,S,128) bf16 buffer.  One tensor per call.
+ * option of dsx_attn_fwd), written to a strided (B,H,S,128) bf16 view; `out` may be `x` itself
+ * (in place).  One tensor per call.
  * Replaces RMSNorm.forward (transformer_helper.py:73-78) followed by apply_rope (flux_dit.py:154-159).
  */
 int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss, const void* norm_w,
