@@ -17,6 +17,7 @@
 // LDS per stage: K tile [64 keys][128 d] (256-byte rows, 16-byte chunk c of row r stored at
 // c ^ (r & 15)) and V^T tile [128 d][64 key slots] (128-byte rows, chunk c of row r stored at
 // c ^ ((r/2) & 7)); both swizzles make 16 consecutive rows at one logical chunk conflict-free.
+#include "attn_internal.h"
 #include "common.h"
 
 namespace dsx {
@@ -416,6 +417,8 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
   if (p->rope && Sq != Skv) return DSX_EBADSHAPE;  // fused RoPE is defined for self/joint attention
   for (int g = 0; g < 2; ++g)
     if (((uintptr_t)p->q_norm_w[g] & 15) || ((uintptr_t)p->k_norm_w[g] & 15)) return DSX_EALIGN;
+
+  if (!fused) return launch_attn_plain(*p, (hipStream_t)stream);
 
   static bool attr_set = false;
   if (!attr_set) {

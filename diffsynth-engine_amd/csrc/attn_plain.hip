@@ -1,0 +1,281 @@
+// Flash attention forward for gfx950 without fused pre-processing (q and k already normalised
+// and rotated): head dim 128, bf16 operands, fp32 online softmax.
+//
+// MFMA formulation as in attn_fwd.hip (S^T = K Q^T, O^T += V^T P^T, one query per lane, so the
+// softmax statistics are lane-local apart from one exchange between the two half-waves).
+//
+// Work split: one workgroup = 8 waves = 256 consecutive queries of one (batch, head); every wave
+// owns 32 queries and needs ~150 VGPRs, so two waves share a SIMD: while one wave's VALU works
+// through exp2/convert/row-sum, the other wave's MFMAs keep the matrix pipe busy.  That costs one
+// LDS operand read per MFMA (128 B/clk per CU at full MFMA rate), which the 256 B/clk LDS of CDNA4
+// carries at half load.
+//
+//  * K and V blocks (64 keys) go HBM/L2 -> LDS with global_load_lds_dwordx4, three stages deep,
+//    both stored row-major [key][128 d].  No staging registers, no transposing stores.
+//  * The V^T operand (8 keys of one d per lane) is read from the row-major V tile with
+//    ds_read_b64_tr_b16: in a 16-lane group, lane i receives element i%4 of the 8-byte datum
+//    addressed by lanes i/4, i/4+4, i/4+8, i/4+12.  Source lane j therefore points at
+//    V[key0 + j/4][d0 + 4*(j%4)], and the receiver gets 4 consecutive keys of d = d0 + i.
+//  * Q is pre-multiplied by softmax_scale*log2(e) once, so P = exp2(S - m_ref) needs no multiply.
+//    The reference m_ref stays 0 (no subtract either) unless a block maximum leaves [-64, 64] in
+//    the first block or exceeds 64 later; after RMSNorm the log2-domain scores are bounded by
+//    128*scale*log2(e) ~ 16.  Moving the reference rescales O and l, so the result is exact
+//    softmax in every case.
+//
+// LDS swizzles: K rows (256 B): 16-byte chunk c of key r at c ^ (r & 15)  (ds_read_b128 by 32 rows);
+//               V rows (256 B): chunk c of key r at c ^ ((r & 3) << 2)    (transposing 8-byte reads).
+#include "attn_internal.h"
+#include "common.h"
+
+namespace dsx {
+
+namespace {
+
+constexpr int QB = 256;  // queries per workgroup (8 waves x 32)
+constexpr int KB = 64;   // keys per block
+constexpr int HD = 128;
+constexpr int kTile = KB * HD * 2;      // 16 KiB
+constexpr int kStage = 2 * kTile;       // K + V
+constexpr int kStages = 3;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kRescaleThreshold = 64.0f;  // log2 units
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int k_off(int key, int chunk) { return key * 256 + ((chunk ^ (key & 15)) << 4); }
+__device__ __forceinline__ int v_off(int key, int chunk) {
+  return key * 256 + ((chunk ^ ((key & 3) << 2)) << 4);
+}
+
+__device__ __forceinline__ float pair_max(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float pair_sum(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+
+__global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;  // 0..7
+  const int g = lane >> 5, li = lane & 31;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int64_t Sq = p.sq[0] + p.sq[1];
+  const int64_t Skv = p.skv[0] + p.skv[1];
+  const int64_t q0 = (int64_t)blockIdx.x * QB + wave * 32;
+
+  const uint16_t* qbase[2];
+  const uint8_t* kbase[2];
+  const uint8_t* vbase[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    qbase[s] = (const uint16_t*)p.q[s] + (int64_t)b * p.q_sb[s] + (int64_t)h * p.q_sh[s];
+    kbase[s] = (const uint8_t*)((const uint16_t*)p.k[s] + (int64_t)b * p.k_sb[s] + (int64_t)h * p.k_sh[s]);
+    vbase[s] = (const uint8_t*)((const uint16_t*)p.v[s] + (int64_t)b * p.v_sb[s] + (int64_t)h * p.v_sh[s]);
+  }
+
+  // ---- async K/V block loads.  One wave instruction = 1 KiB = 4 keys x 256 B; lane l lands at key
+  //      l/16, physical chunk l%16.  Per block a wave issues 2 K and 2 V instructions (8 keys).
+  const int ld_r = lane >> 4, ld_p = lane & 15;
+  auto issue_block = [&](int kb, int stage) {
+    uint8_t* sK = smem + stage * kStage + wave * 2 * 1024;
+    uint8_t* sV = sK + kTile;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = (wave * 2 + i) * 4 + ld_r;
+      int64_t key = (int64_t)kb * KB + row;
+      if (key >= Skv) key = Skv - 1;
+      const int seg = key >= p.skv[0] ? 1 : 0;
+      const int64_t lrow = key - (seg ? p.skv[0] : 0);
+      const int ck = ld_p ^ (row & 15);
+      const int cv = ld_p ^ ((row & 3) << 2);
+      __builtin_amdgcn_global_load_lds((gptr_t)(kbase[seg] + lrow * p.k_ss[seg] * 2 + ck * 16),
+                                       (lptr_t)(sK + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(vbase[seg] + lrow * p.v_ss[seg] * 2 + cv * 16),
+                                       (lptr_t)(sV + i * 1024), 16, 0, 0);
+    }
+  };
+
+  const int nkb = (int)((Skv + KB - 1) / KB);
+  issue_block(0, 0);
+  issue_block(min(1, nkb - 1), 1);
+
+  // ---- Q fragments (B operand of S^T = K Q^T), pre-multiplied by scale*log2(e)
+  const float c = p.softmax_scale * kLog2e;
+  bf16x8 qf[8];
+  {
+    int64_t row = q0 + li;
+    if (row >= Sq) row = Sq - 1;
+    const int seg = row >= p.sq[0] ? 1 : 0;
+    const uint16_t* src = qbase[seg] + (row - (seg ? p.sq[0] : 0)) * p.q_ss[seg];
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(src + kc * 16 + g * 8);
+      u32x4 sc;
+      sc.x = pack_bf16x2(bf16_lo(raw.x) * c, bf16_hi(raw.x) * c);
+      sc.y = pack_bf16x2(bf16_lo(raw.y) * c, bf16_hi(raw.y) * c);
+      sc.z = pack_bf16x2(bf16_lo(raw.z) * c, bf16_hi(raw.z) * c);
+      sc.w = pack_bf16x2(bf16_lo(raw.w) * c, bf16_hi(raw.w) * c);
+      qf[kc] = __builtin_bit_cast(bf16x8, sc);
+    }
+  }
+
+  f32x16 oacc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float m_ref = 0.f;     // softmax reference of the lane's query (log2 domain)
+  bool any_ref = false;  // wave-uniform: some lane of this wave has m_ref != 0
+  float l_run = 0.f;
+
+  // transposing V reads: source-lane role of this lane inside its 16-lane group
+  const int grp = lane >> 4, j16 = lane & 15;
+  const int tr_key = ((grp >> 1) << 2) + (j16 >> 2);    // 4*g of the receiving lanes + key within the quad
+  const int tr_dbyte = (grp & 1) * 32 + (j16 & 3) * 8;  // + dt*64, bytes within the 256-byte row
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  for (int kb = 0; kb < nkb; ++kb) {
+    const int stage = kb % kStages;
+    // block kb has landed once at most the 4 loads of block kb+1 are still in flight; the barrier
+    // also tells that every wave is done with block kb-1, whose stage block kb+2 will overwrite
+    __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+    __builtin_amdgcn_s_barrier();
+    issue_block(min(kb + 2, nkb - 1), (kb + 2) % kStages);
+    const uint8_t* sK = smem + stage * kStage;
+    const uint8_t* sV = sK + kTile;
+
+    // ---- S^T = K (cQ)^T for the 64 keys of the block: two 32-key tiles
+    f32x16 s[2];
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + k_off(kt * 32 + li, 2 * kc + g));
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kc], kc == 0 ? zero16 : s[kt], 0, 0, 0);
+      }
+    }
+    if ((int64_t)(kb + 1) * KB > Skv) {  // ragged tail of the key axis
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t key = (int64_t)kb * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (key >= Skv) s[kt][r] = -INFINITY;
+        }
+    }
+    if (any_ref) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[kt][r] -= m_ref;
+    }
+    // ---- block maximum relative to the reference; move the reference only when it must move
+    float m0 = max3(s[0][0], s[0][1], s[0][2]);
+    float m1 = max3(s[1][0], s[1][1], s[1][2]);
+#pragma unroll
+    for (int r = 3; r < 15; r += 2) {
+      m0 = max3(m0, s[0][r], s[0][r + 1]);
+      m1 = max3(m1, s[1][r], s[1][r + 1]);
+    }
+    const float mx = pair_max(max3(m0, m1, fmaxf(s[0][15], s[1][15])));
+    const bool move = mx > kRescaleThreshold || (kb == 0 && mx < -kRescaleThreshold);
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      any_ref = true;
+      const float d = kb == 0 ? mx : fmaxf(mx, 0.f);
+      const float alpha = kb == 0 ? 1.0f : __builtin_amdgcn_exp2f(-d);
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[kt][r] -= d;
+      m_ref += d;
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    }
+
+    // ---- P = exp2(S'), packed to bf16; the row sum is taken over the ROUNDED values (v_dot2 with
+    //      ones), i.e. over exactly the numbers the PV product uses
+    uint32_t pw[2][8];  // [kt][word]: entries 2w, 2w+1
+    float lsum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int w = 0; w < 8; ++w) {
+        const float p0 = __builtin_amdgcn_exp2f(s[kt][2 * w]);
+        const float p1 = __builtin_amdgcn_exp2f(s[kt][2 * w + 1]);
+        pw[kt][w] = pack_bf16x2(p0, p1);
+        lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pw[kt][w]), ones2, lsum, false);
+      }
+    l_run += lsum;
+
+    // ---- O^T += V^T P^T.  16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int ch = 0; ch < 2; ++ch) {
+        const int key0 = kt * 32 + ch * 16 + tr_key;
+        const u32x4 w = {pw[kt][4 * ch + 0], pw[kt][4 * ch + 1], pw[kt][4 * ch + 2], pw[kt][4 * ch + 3]};
+        const bf16x8 pf = __builtin_bit_cast(bf16x8, w);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+          const int dbyte = dt * 64 + tr_dbyte;
+          const int chunk = dbyte >> 4, within = dbyte & 15;
+          const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) v4i16*)(sV + v_off(key0, chunk) + within));
+          const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (__attribute__((address_space(3))) v4i16*)(sV + v_off(key0 + 8, chunk) + within));
+          typedef short v8i16 __attribute__((ext_vector_type(8)));
+          const v8i16 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, oacc[dt], 0, 0, 0);
+        }
+      }
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // drain trailing async loads
+
+  // ---- normalise and store.  lane (g, j): query j, d = dt*32 + 8*(r/4) + 4g + r%4
+  const float inv = 1.0f / pair_sum(l_run);
+  const int64_t row = q0 + li;
+  if (row < Sq) {
+    const int seg = row >= p.sq[0] ? 1 : 0;
+    uint16_t* dst = (uint16_t*)p.o[seg] + (int64_t)b * p.o_sb[seg] + (int64_t)h * p.o_sh[seg] +
+                    (row - (seg ? p.sq[0] : 0)) * p.o_ss[seg];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        u32x2 w;
+        w.x = pack_bf16x2(oacc[dt][4 * rq + 0] * inv, oacc[dt][4 * rq + 1] * inv);
+        w.y = pack_bf16x2(oacc[dt][4 * rq + 2] * inv, oacc[dt][4 * rq + 3] * inv);
+        *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w;
+      }
+  }
+}
+
+}  // namespace
+
+int launch_attn_plain(const dsx_attn_params& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)attn_plain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kStages * kStage) != hipSuccess)
+      return DSX_ELAUNCH;
+    attr_set = true;
+  }
+  const int64_t Sq = p.sq[0] + p.sq[1];
+  dim3 grid((unsigned)((Sq + QB - 1) / QB), (unsigned)p.heads, (unsigned)p.batch), block(512);
+  attn_plain_kernel<<<grid, block, kStages * kStage, st>>>(p);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+}  // namespace dsx
