@@ -57,6 +57,13 @@ SIGNATURES = {
     "dsx_cast_fp8_scaled": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "dsx_fp8_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                              c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "dsx_fp8_gemm_gated_residual": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
+                                            c_int64, c_int64, c_int64, c_void_p]),
+    "dsx_fp8_gemv_rowscale": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "dsx_concat_gelu_tanh": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
+                                     c_int64, c_void_p, c_int64, c_int64, c_void_p]),
     "dsx_attn_fwd": (c_int, [ctypes.POINTER(AttnParams), c_void_p]),
     "dsx_rmsnorm_rope": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int64,
                                  c_int64, c_void_p, c_int64, c_int64, c_int64, ctypes.c_int32, ctypes.c_int32,

@@ -1,22 +1,29 @@
 // Bandwidth-bound row kernels of the DiT block: AdaLN modulate (LayerNorm + scale/shift),
-// gated residual, tanh-GELU, flow-match Euler update.  One workgroup of 256 threads owns one
-// row, keeps it in registers (16-byte loads, 8 bf16 per chunk), reduces through the wavefront
-// and a 4-entry LDS exchange, and can emit the row as bf16 and/or as per-token-scaled e4m3
-// (the operand format of the following FP8 GEMM) in the same pass.
+// gated residual, tanh-GELU (optionally concatenated behind an untouched prefix), flow-match Euler
+// update.  A wavefront (rows up to 6144 wide) or a workgroup of 256 threads owns one row, keeps it in
+// registers (16-byte loads, 8 bf16 per chunk), reduces through the wavefront (plus a 4-entry LDS
+// exchange for workgroup rows), and can emit the row as bf16 and/or as per-token-scaled e4m3 (the
+// operand format of the following FP8 GEMM) in the same pass.
 #include "common.h"
 
 namespace dsx {
 
-__device__ __forceinline__ float block_sum(float v, float* red) {
+// Row reductions for TPR threads per row: TPR == 64 is one wavefront per row (four rows per
+// workgroup, no LDS, no barrier); TPR == 256 is the whole workgroup on one row.
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float* red) {
   v = wave_sum(v);
+  if (TPR == 64) return v;
   const int w = threadIdx.x >> 6;
   __syncthreads();  // protect `red` against a previous reduction still being read
   if ((threadIdx.x & 63) == 0) red[w] = v;
   __syncthreads();
   return red[0] + red[1] + red[2] + red[3];
 }
-__device__ __forceinline__ float block_max(float v, float* red) {
+template <int TPR>
+__device__ __forceinline__ float row_max(float v, float* red) {
   v = wave_max(v);
+  if (TPR == 64) return v;
   const int w = threadIdx.x >> 6;
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[w] = v;
@@ -30,10 +37,10 @@ __device__ __forceinline__ void unpack8(const u32x4& w, float* v) {
 }
 __device__ __forceinline__ u32x4 pack8(const float* v) {
   u32x4 o;
-  o.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-  o.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
-  o.z = f32_to_bf16_bits(v[4]) | (f32_to_bf16_bits(v[5]) << 16);
-  o.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
+  o.x = pack_bf16x2(v[0], v[1]);
+  o.y = pack_bf16x2(v[2], v[3]);
+  o.z = pack_bf16x2(v[4], v[5]);
+  o.w = pack_bf16x2(v[6], v[7]);
   return o;
 }
 __device__ __forceinline__ u32x2 quant8(const float* v, float inv) {
@@ -47,14 +54,14 @@ __device__ __forceinline__ u32x2 quant8(const float* v, float inv) {
 }
 
 // Emit a row held as NCH register chunks of 8 already-bf16-rounded floats.
-template <int NCH>
+template <int NCH, int TPR>
 __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint16_t* y, uint8_t* q,
                                          float* q_scale, int64_t row, float* red) {
-  const int tid = threadIdx.x;
+  const int t = threadIdx.x % TPR;
   if (y) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = tid + i * 256;
+      const int c = t + i * TPR;
       if (c < nchunk) reinterpret_cast<u32x4*>(y)[c] = pack8(val[i]);
     }
   }
@@ -62,41 +69,42 @@ __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint1
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = tid + i * 256;
+      const int c = t + i * TPR;
       if (c < nchunk) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(val[i][j]));
       }
     }
-    amax = block_max(amax, red);
-    amax = fmaxf(amax, 1e-12f);
+    amax = fmaxf(row_max<TPR>(amax, red), 1e-12f);
     const float inv = 448.0f / amax;
-    if (tid == 0) q_scale[row] = amax / 448.0f;
+    if (t == 0) q_scale[row] = amax / 448.0f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = tid + i * 256;
+      const int c = t + i * TPR;
       if (c < nchunk) reinterpret_cast<u32x2*>(q)[c] = quant8(val[i], inv);
     }
   }
 }
 
-template <int NCH>
+template <int NCH, int TPR>
 __global__ __launch_bounds__(256) void adaln_modulate_kernel(
     const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ scale,
     const uint16_t* __restrict__ shift, int64_t mod_sb, int64_t rows_per_batch,
     const uint16_t* __restrict__ ln_w, const uint16_t* __restrict__ ln_b, float eps,
     uint16_t* __restrict__ y, int64_t ldy, uint8_t* __restrict__ q, int64_t ldq,
-    float* __restrict__ q_scale, int D) {
+    float* __restrict__ q_scale, int64_t rows, int D) {
   __shared__ float red[4];
-  const int tid = threadIdx.x;
-  const int64_t row = blockIdx.x;
+  const int t = threadIdx.x % TPR;
+  int64_t row = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
+  const bool live = row < rows;  // only possible to fail for TPR == 64 (whole wavefront idle)
+  if (!live) row = rows - 1;
   const int nchunk = D >> 3;
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
   float val[NCH][8];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = tid + i * 256;
+    const int c = t + i * TPR;
     if (c < nchunk) {
       u32x4 w = xr[c];
       unpack8(w, val[i]);
@@ -104,11 +112,11 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
       for (int j = 0; j < 8; ++j) sum += val[i][j];
     }
   }
-  const float mean = block_sum(sum, red) / (float)D;
+  const float mean = row_sum<TPR>(sum, red) / (float)D;
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = tid + i * 256;
+    const int c = t + i * TPR;
     if (c < nchunk) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -117,13 +125,13 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
       }
     }
   }
-  const float rstd = rsqrtf(block_sum(sq, red) / (float)D + eps);
+  const float rstd = rsqrtf(row_sum<TPR>(sq, red) / (float)D + eps);
   const int64_t bidx = row / rows_per_batch;
   const u32x4* sc = scale ? reinterpret_cast<const u32x4*>(scale + bidx * mod_sb) : nullptr;
   const u32x4* sh = shift ? reinterpret_cast<const u32x4*>(shift + bidx * mod_sb) : nullptr;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = tid + i * 256;
+    const int c = t + i * TPR;
     if (c < nchunk) {
       float v[8];
 #pragma unroll
@@ -158,33 +166,44 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
       for (int j = 0; j < 8; ++j) val[i][j] = v[j];
     }
   }
-  emit_row<NCH>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
-                red);
+  if (!live) return;  // wave-uniform
+  emit_row<NCH, TPR>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
+                     red);
 }
 
+// tanh-GELU of x, optionally preceded in the OUTPUT row by an unmodified prefix:
+// out row = [ prefix (Dp) | gelu(x) (D) ].  The prefix form is the single-stream block's
+// cat([attention, gelu(mlp)]) built directly in the operand format of proj_out.
 template <int NCH>
-__global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restrict__ prefix, int64_t ldp,
+                                                        int Dp, const uint16_t* __restrict__ x, int64_t ldx,
                                                         uint16_t* __restrict__ y, int64_t ldy,
                                                         uint8_t* __restrict__ q, int64_t ldq,
                                                         float* __restrict__ q_scale, int D) {
   __shared__ float red[4];
   const int tid = threadIdx.x;
   const int64_t row = blockIdx.x;
-  const int nchunk = D >> 3;
+  const int npre = Dp >> 3;
+  const int nchunk = npre + (D >> 3);
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  const u32x4* pr = reinterpret_cast<const u32x4*>(prefix + row * ldp);
   float val[NCH][8];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = tid + i * 256;
     if (c < nchunk) {
-      u32x4 w = __builtin_nontemporal_load(xr + c);
-      unpack8(w, val[i]);
+      if (c < npre) {
+        unpack8(pr[c], val[i]);
+      } else {
+        u32x4 w = __builtin_nontemporal_load(xr + (c - npre));
+        unpack8(w, val[i]);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(gelu_tanh_f32(val[i][j]));
+        for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(gelu_tanh_f32(val[i][j]));
+      }
     }
   }
-  emit_row<NCH>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
-                red);
+  emit_row<NCH, 256>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
+                     red);
 }
 
 __global__ __launch_bounds__(256) void gated_residual_kernel(
@@ -252,16 +271,35 @@ extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale,
     return DSX_EALIGN;
   if (rows == 0) return DSX_OK;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)rows), block(256);
-#define DSX_LAUNCH_ADALN(NCH)                                                                     \
-  adaln_modulate_kernel<NCH><<<grid, block, 0, st>>>(                                             \
-      (const uint16_t*)x, ldx, (const uint16_t*)scale, (const uint16_t*)shift, mod_sb,            \
-      rows_per_batch, (const uint16_t*)ln_w, (const uint16_t*)ln_b, eps, (uint16_t*)y, ldy,       \
-      (uint8_t*)q, ldq, q_scale, (int)D)
-  if (D <= 2048 * 2) DSX_LAUNCH_ADALN(2);
-  else if (D <= 2048 * 3) DSX_LAUNCH_ADALN(3);
-  else DSX_LAUNCH_ADALN(8);
+  dim3 block(256);
+#define DSX_LAUNCH_ADALN(NCH, TPR)                                                                 \
+  adaln_modulate_kernel<NCH, TPR><<<dim3((unsigned)((rows + 256 / TPR - 1) / (256 / TPR))), block, 0, st>>>( \
+      (const uint16_t*)x, ldx, (const uint16_t*)scale, (const uint16_t*)shift, mod_sb,             \
+      rows_per_batch, (const uint16_t*)ln_w, (const uint16_t*)ln_b, eps, (uint16_t*)y, ldy,        \
+      (uint8_t*)q, ldq, q_scale, rows, (int)D)
+  // one wavefront per row while a row fits 12 chunks per lane and there are rows enough to fill the chip
+  if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_ADALN(6, 64);
+  else if (D <= 512 * 12 && rows >= 1024) DSX_LAUNCH_ADALN(12, 64);
+  else if (D <= 2048 * 2) DSX_LAUNCH_ADALN(2, 256);
+  else if (D <= 2048 * 3) DSX_LAUNCH_ADALN(3, 256);
+  else DSX_LAUNCH_ADALN(8, 256);
 #undef DSX_LAUNCH_ADALN
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+static int launch_gelu(const void* prefix, int64_t ldp, int64_t Dp, const void* x, int64_t ldx, void* y,
+                       int64_t ldy, void* q, int64_t ldq, float* q_scale, int64_t rows, int64_t D,
+                       hipStream_t st) {
+  using namespace dsx;
+  const int64_t Dt = Dp + D;
+  dim3 grid((unsigned)rows), block(256);
+#define DSX_LAUNCH_GELU(NCH)                                                                        \
+  gelu_tanh_kernel<NCH><<<grid, block, 0, st>>>((const uint16_t*)prefix, ldp, (int)Dp, (const uint16_t*)x, \
+                                                ldx, (uint16_t*)y, ldy, (uint8_t*)q, ldq, q_scale, (int)D)
+  if (Dt <= 2048 * 2) DSX_LAUNCH_GELU(2);
+  else if (Dt <= 2048 * 6) DSX_LAUNCH_GELU(6);
+  else DSX_LAUNCH_GELU(8);
+#undef DSX_LAUNCH_GELU
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
@@ -275,16 +313,23 @@ extern "C" int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, v
       ((uintptr_t)q & 7))
     return DSX_EALIGN;
   if (rows == 0) return DSX_OK;
-  hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)rows), block(256);
-#define DSX_LAUNCH_GELU(NCH)                                                                  \
-  gelu_tanh_kernel<NCH><<<grid, block, 0, st>>>((const uint16_t*)x, ldx, (uint16_t*)y, ldy,   \
-                                                (uint8_t*)q, ldq, q_scale, (int)D)
-  if (D <= 2048 * 2) DSX_LAUNCH_GELU(2);
-  else if (D <= 2048 * 6) DSX_LAUNCH_GELU(6);
-  else DSX_LAUNCH_GELU(8);
-#undef DSX_LAUNCH_GELU
-  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+  return launch_gelu(x, 0, 0, x, ldx, y, ldy, q, ldq, q_scale, rows, D, (hipStream_t)stream);
+}
+
+extern "C" int dsx_concat_gelu_tanh(const void* prefix, int64_t ldp, int64_t Dp, const void* x, int64_t ldx,
+                                    void* y, int64_t ldy, void* q, int64_t ldq, float* q_scale,
+                                    int64_t rows, int64_t D, void* stream) {
+  using namespace dsx;
+  if (!prefix || !x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
+  const int64_t Dt = Dp + D;
+  if (rows < 0 || D <= 0 || Dp <= 0 || (D & 7) || (Dp & 7) || Dt > 16384 || ldx < D || ldp < Dp ||
+      (y && ldy < Dt) || (q && ldq < Dt))
+    return DSX_EBADSHAPE;
+  if ((ldx & 7) || (ldp & 7) || (y && (ldy & 7)) || (q && (ldq & 7)) || misaligned16(x) ||
+      misaligned16(prefix) || misaligned16(y) || ((uintptr_t)q & 7))
+    return DSX_EALIGN;
+  if (rows == 0) return DSX_OK;
+  return launch_gelu(prefix, ldp, Dp, x, ldx, y, ldy, q, ldq, q_scale, rows, D, (hipStream_t)stream);
 }
 
 extern "C" int dsx_gated_residual(const void* x, int64_t ldx, const void* y, int64_t ldy,

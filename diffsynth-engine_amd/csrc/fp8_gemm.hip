@@ -37,6 +37,13 @@ struct GemmArgs {
   int64_t lda, ldw, ldo;
   int M, N, K;
   int tiles_m, tiles_n;
+  // optional fused gated residual: out = resid + gate * bf16(acc*scale + bias)
+  const uint16_t* resid;
+  const uint16_t* gate;  // (N,) per batch entry, batch = row / rows_per_batch; NULL = gate of 1
+  int64_t ldr, gate_sb;
+  int rows_per_batch;
+  // optional per-output-row weight scale (GEMV path only)
+  const float* w_row_scale;
 };
 
 __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn,
@@ -59,6 +66,14 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
+
+// resid + bf16(gate * proj) for one element; proj is already rounded to bf16.
+__device__ __forceinline__ float residual_combine(const GemmArgs& p, float proj, int m, int n) {
+  const float rv = bf16_bits_to_f32(p.resid[(int64_t)m * p.ldr + n]);
+  if (p.gate)
+    proj = round_bf16(bf16_bits_to_f32(p.gate[(int64_t)(m / p.rows_per_batch) * p.gate_sb + n]) * proj);
+  return rv + proj;
+}
 
 // Store one C^T accumulator tile set of a wave.  acc[tn][tm]: rows n, columns m (see header).
 __device__ __forceinline__ void store_ct(const GemmArgs& p, f32x16 (&acc)[4][4], int n_base,
@@ -84,8 +99,14 @@ __device__ __forceinline__ void store_ct(const GemmArgs& p, f32x16 (&acc)[4][4],
               b0 = bf16_lo(bw.x); b1 = bf16_hi(bw.x); b2 = bf16_lo(bw.y); b3 = bf16_hi(bw.y);
             }
             u32x2 o;
-            o.x = pack_bf16x2(acc[tn][tm][4 * rq + 0] * sc + b0, acc[tn][tm][4 * rq + 1] * sc + b1);
-            o.y = pack_bf16x2(acc[tn][tm][4 * rq + 2] * sc + b2, acc[tn][tm][4 * rq + 3] * sc + b3);
+            float r[4] = {acc[tn][tm][4 * rq + 0] * sc + b0, acc[tn][tm][4 * rq + 1] * sc + b1,
+                          acc[tn][tm][4 * rq + 2] * sc + b2, acc[tn][tm][4 * rq + 3] * sc + b3};
+            if (p.resid) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) r[e] = residual_combine(p, round_bf16(r[e]), m, n + e);
+            }
+            o.x = pack_bf16x2(r[0], r[1]);
+            o.y = pack_bf16x2(r[2], r[3]);
             *reinterpret_cast<u32x2*>(orow + n) = o;
           }
         } else {
@@ -93,7 +114,9 @@ __device__ __forceinline__ void store_ct(const GemmArgs& p, f32x16 (&acc)[4][4],
           for (int e = 0; e < 4; ++e) {
             if (n + e < p.N) {
               const float bj = p.bias ? bf16_bits_to_f32(p.bias[n + e]) : 0.f;
-              orow[n + e] = (uint16_t)f32_to_bf16_bits(acc[tn][tm][4 * rq + e] * sc + bj);
+              float r = acc[tn][tm][4 * rq + e] * sc + bj;
+              if (p.resid) r = residual_combine(p, round_bf16(r), m, n + e);
+              orow[n + e] = (uint16_t)f32_to_bf16_bits(r);
             }
           }
         }
@@ -133,6 +156,7 @@ __device__ __forceinline__ void load_epi_operands(const GemmArgs& p, EpiOperands
   }
 }
 
+template <bool RESID>
 __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][4], const EpiOperands& e,
                                              uint8_t* wave_lds, int n_base, int m_base, int lane) {
   const int g = lane >> 5, li = lane & 31;
@@ -163,9 +187,24 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
 #pragma unroll
   for (int it = 0; it < 32; ++it) {
     const int ml = it * 4 + r0;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
-    if (m_base + ml < p.M && n < p.N)
-      *reinterpret_cast<u32x4*>(p.out + (int64_t)(m_base + ml) * p.ldo + n) = v;
+    u32x4 v = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
+    const int m = m_base + ml;
+    if (m < p.M && n < p.N) {
+      if (RESID) {
+        // rounding points of the separate ops: bf16(gate * proj), then bf16(resid + .)
+        const u32x4 rv = *reinterpret_cast<const u32x4*>(p.resid + (int64_t)m * p.ldr + n);
+        u32x4 gv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+        if (p.gate)
+          gv = *reinterpret_cast<const u32x4*>(p.gate + (int64_t)(m / p.rows_per_batch) * p.gate_sb + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float t0 = p.gate ? round_bf16(bf16_lo(gv[e]) * bf16_lo(v[e])) : bf16_lo(v[e]);
+          const float t1 = p.gate ? round_bf16(bf16_hi(gv[e]) * bf16_hi(v[e])) : bf16_hi(v[e]);
+          v[e] = pack_bf16x2(bf16_lo(rv[e]) + t0, bf16_hi(rv[e]) + t1);
+        }
+      }
+      *reinterpret_cast<u32x4*>(p.out + (int64_t)m * p.ldo + n) = v;
+    }
   }
 }
 
@@ -185,6 +224,7 @@ __device__ __forceinline__ int slab_off(int row, int chunk) {
   return row * SK + ((chunk ^ ((row >> 2) & 3)) << 4);
 }
 
+template <bool RESID>
 __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int tm, tn;
@@ -293,20 +333,16 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is reused
 
-  const bool vec_ok = ((p.ldo & 7) == 0) && ((p.N & 7) == 0) && (((uintptr_t)p.out & 15) == 0) &&
-                      (!p.bias || ((uintptr_t)p.bias & 7) == 0);
-  if (vec_ok) {
-    EpiOperands epi;
-    load_epi_operands(p, epi, n0 + wn * 128, m0 + wm * 128, lane);
-    __syncthreads();  // every wave is done reading the operand stages
-    store_ct_lds(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 128, lane);
-  } else {
-    store_ct(p, acc, n0 + wn * 128, m0 + wm * 128, g, li);
-  }
+  // (the launcher sends shapes the vectorised epilogue cannot store to the generic kernel)
+  EpiOperands epi;
+  load_epi_operands(p, epi, n0 + wn * 128, m0 + wm * 128, lane);
+  __syncthreads();  // every wave is done reading the operand stages
+  store_ct_lds<RESID>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 128, lane);
 }
 
 // ------------------------------------------------------------------------------------------
-// Generic kernel for K % 128 != 0 (K % 16 == 0): register-staged loads with a zero-filled K tail.
+// Generic kernel: any K % 16 == 0 (zero-filled K tail), any N / alignment (scalar stores where the
+// 8-byte path does not apply).  Register-staged loads, one LDS stage; used for the few odd shapes.
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fp8_gemm_ragged_k_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -374,60 +410,125 @@ __global__ __launch_bounds__(256) void fp8_gemm_ragged_k_kernel(GemmArgs p) {
   store_ct(p, acc, n0 + wn * 128, m0 + wm * 128, g, li);
 }
 
-// Small-M path (M <= 8): one wave per output column, fp32 FMA over dequantised bytes.
-// HBM-bound on the weight read; used for the M=1 conditioning projections.
+// Small-M path (M <= 8): HBM-bound on the weight read (the M=1 conditioning projections).
+// One wavefront owns four output rows; per K chunk of 1 KiB a lane fetches 16 weight bytes of
+// each row (four independent loads in flight) and reuses its 16 activation bytes per token.
+// fp32 FMA over the dequantised bytes; the per-row scale form serves several Linear layers
+// stacked into one weight matrix.
+__device__ __forceinline__ void dequant16(const u32x4& v, float* f) {
+#pragma unroll
+  for (int b = 0; b < 16; ++b) f[b] = e4m3_bits_to_f32((v[b >> 2] >> ((b & 3) * 8)) & 0xffu);
+}
+
+template <int MT>
 __global__ __launch_bounds__(256) void fp8_gemv_kernel(GemmArgs p) {
   const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= p.N) return;
+  const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 4;
+  if (n0 >= p.N) return;
   const int kchunks = p.K >> 4;
-  float acc[8];
+  float acc[4][MT];
 #pragma unroll
-  for (int m = 0; m < 8; ++m) acc[m] = 0.f;
-  const u32x4* wr = reinterpret_cast<const u32x4*>(p.w + (int64_t)n * p.ldw);
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
+  const u32x4* wr[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) wr[r] = reinterpret_cast<const u32x4*>(p.w + (int64_t)min(n0 + r, p.N - 1) * p.ldw);
   for (int c = lane; c < kchunks; c += 64) {
-    u32x4 wv = __builtin_nontemporal_load(wr + c);
-    float wf[16];
+    u32x4 wv[4];
 #pragma unroll
-    for (int b = 0; b < 16; ++b) wf[b] = e4m3_bits_to_f32((wv[b >> 2] >> ((b & 3) * 8)) & 0xffu);
+    for (int r = 0; r < 4; ++r) wv[r] = __builtin_nontemporal_load(wr[r] + c);
+    float af[MT][16];
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-      if (m < p.M) {
-        u32x4 av = *reinterpret_cast<const u32x4*>(p.a + (int64_t)m * p.lda + c * 16);
+    for (int m = 0; m < MT; ++m) {
+      const u32x4 av = *reinterpret_cast<const u32x4*>(p.a + (int64_t)min(m, p.M - 1) * p.lda + c * 16);
+      dequant16(av, af[m]);
+    }
 #pragma unroll
-        for (int b = 0; b < 16; ++b)
-          acc[m] += wf[b] * e4m3_bits_to_f32((av[b >> 2] >> ((b & 3) * 8)) & 0xffu);
-      }
+    for (int r = 0; r < 4; ++r) {
+      float wf[16];
+      dequant16(wv[r], wf);
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int b = 0; b < 16; ++b) acc[r][m] += wf[b] * af[m][b];
     }
   }
   const float ws = p.w_scale ? *p.w_scale : 1.0f;
-  const float bj = p.bias ? bf16_bits_to_f32(p.bias[n]) : 0.f;
 #pragma unroll
-  for (int m = 0; m < 8; ++m) {
-    if (m < p.M) {
-      float s = wave_sum(acc[m]);
-      if (lane == 0) {
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + r;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const float s = wave_sum(acc[r][m]);
+      if (lane == 0 && n < p.N && m < p.M) {
         const float as = p.a_scale ? p.a_scale[m] : 1.0f;
-        p.out[(int64_t)m * p.ldo + n] = (uint16_t)f32_to_bf16_bits(s * (as * ws) + bj);
+        const float wsn = p.w_row_scale ? p.w_row_scale[n] : ws;
+        const float bj = p.bias ? bf16_bits_to_f32(p.bias[n]) : 0.f;
+        float r = s * (as * wsn) + bj;
+        if (p.resid) r = residual_combine(p, round_bf16(r), m, n);
+        p.out[(int64_t)m * p.ldo + n] = (uint16_t)f32_to_bf16_bits(r);
       }
     }
   }
 }
 
+static int launch_gemv(const GemmArgs& p, hipStream_t st) {
+  const dim3 grid((unsigned)((p.N + 15) / 16)), block(256);
+  if (p.M == 1) fp8_gemv_kernel<1><<<grid, block, 0, st>>>(p);
+  else if (p.M == 2) fp8_gemv_kernel<2><<<grid, block, 0, st>>>(p);
+  else if (p.M <= 4) fp8_gemv_kernel<4><<<grid, block, 0, st>>>(p);
+  else fp8_gemv_kernel<8><<<grid, block, 0, st>>>(p);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
 }  // namespace dsx
 
-extern "C" int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t ldw,
-                            const float* a_scale, const float* w_scale, const void* bias, void* out,
-                            int64_t ldo, int64_t M, int64_t N, int64_t K, void* stream) {
+static int gemm_dispatch(dsx::GemmArgs& p, int64_t M, int64_t N, int64_t K, hipStream_t st) {
   using namespace dsx;
+  if (M <= 8) {
+    p.tiles_m = p.tiles_n = 0;
+    return launch_gemv(p, st);
+  }
+  if (p.w_row_scale) return DSX_EBADSHAPE;
+  p.tiles_m = (int)((M + BM - 1) / BM);
+  p.tiles_n = (int)((N + BN - 1) / BN);
+  const int total = p.tiles_m * p.tiles_n;
+  const int grid = ((total + 7) / 8) * 8;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)fp8_gemm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kMainLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kMainLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
+      return DSX_ELAUNCH;
+    attr_set = true;
+  }
+  const bool vec_ok = ((p.ldo & 7) == 0) && ((p.N & 7) == 0) && (((uintptr_t)p.out & 15) == 0) &&
+                      (!p.bias || ((uintptr_t)p.bias & 7) == 0) &&
+                      (!p.resid || ((((uintptr_t)p.resid & 15) == 0) && ((p.ldr & 7) == 0) &&
+                                    (((uintptr_t)p.gate & 15) == 0) && ((p.gate_sb & 7) == 0)));
+  if ((K % 128) == 0 && vec_ok) {
+    if (p.resid)
+      fp8_gemm_kernel<true><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(p);
+    else
+      fp8_gemm_kernel<false><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(p);
+  } else
+    fp8_gemm_ragged_k_kernel<<<dim3((unsigned)grid), dim3(256), kStageBytes, st>>>(p);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+static int gemm_fill(dsx::GemmArgs& p, const void* a, int64_t lda, const void* w, int64_t ldw,
+                     const float* a_scale, const float* w_scale, const void* bias, void* out, int64_t ldo,
+                     int64_t M, int64_t N, int64_t K) {
   if (!a || !w || !out) return DSX_ENULL;
   if (M < 0 || N <= 0 || K <= 0 || (K & 15) || lda < K || ldw < K || ldo < N) return DSX_EBADSHAPE;
   if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return DSX_EBADSHAPE;
   if ((lda & 15) || (ldw & 15) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)out & 1) ||
       ((uintptr_t)bias & 1))
     return DSX_EALIGN;
-  if (M == 0) return DSX_OK;
-  GemmArgs p;
   p.a = (const uint8_t*)a;
   p.w = (const uint8_t*)w;
   p.a_scale = a_scale;
@@ -440,28 +541,52 @@ extern "C" int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t l
   p.M = (int)M;
   p.N = (int)N;
   p.K = (int)K;
-  hipStream_t st = (hipStream_t)stream;
-  if (M <= 8) {
-    p.tiles_m = p.tiles_n = 0;
-    fp8_gemv_kernel<<<dim3((unsigned)((N + 3) / 4)), dim3(256), 0, st>>>(p);
-    return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
-  }
-  p.tiles_m = (int)((M + BM - 1) / BM);
-  p.tiles_n = (int)((N + BN - 1) / BN);
-  const int total = p.tiles_m * p.tiles_n;
-  const int grid = ((total + 7) / 8) * 8;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)fp8_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
-      return DSX_ELAUNCH;
-    attr_set = true;
-  }
-  if ((K % 128) == 0)
-    fp8_gemm_kernel<<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(p);
-  else
-    fp8_gemm_ragged_k_kernel<<<dim3((unsigned)grid), dim3(256), kStageBytes, st>>>(p);
-  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+  p.resid = nullptr;
+  p.gate = nullptr;
+  p.ldr = p.gate_sb = 0;
+  p.rows_per_batch = 1;
+  p.w_row_scale = nullptr;
+  return DSX_OK;
+}
+
+extern "C" int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t ldw,
+                            const float* a_scale, const float* w_scale, const void* bias, void* out,
+                            int64_t ldo, int64_t M, int64_t N, int64_t K, void* stream) {
+  dsx::GemmArgs p;
+  const int rc = gemm_fill(p, a, lda, w, ldw, a_scale, w_scale, bias, out, ldo, M, N, K);
+  if (rc != DSX_OK || M == 0) return rc;
+  return gemm_dispatch(p, M, N, K, (hipStream_t)stream);
+}
+
+extern "C" int dsx_fp8_gemm_gated_residual(const void* a, int64_t lda, const void* w, int64_t ldw,
+                                           const float* a_scale, const float* w_scale, const void* bias,
+                                           const void* resid, int64_t ldr, const void* gate, int64_t gate_sb,
+                                           int64_t rows_per_batch, void* out, int64_t ldo, int64_t M,
+                                           int64_t N, int64_t K, void* stream) {
+  dsx::GemmArgs p;
+  const int rc = gemm_fill(p, a, lda, w, ldw, a_scale, w_scale, bias, out, ldo, M, N, K);
+  if (rc != DSX_OK) return rc;
+  if (!resid) return DSX_ENULL;
+  if (ldr < N || rows_per_batch <= 0 || rows_per_batch > (1 << 30)) return DSX_EBADSHAPE;
+  if (((uintptr_t)resid & 1) || ((uintptr_t)gate & 1)) return DSX_EALIGN;
+  if (M == 0) return DSX_OK;
+  p.resid = (const uint16_t*)resid;
+  p.gate = (const uint16_t*)gate;
+  p.ldr = ldr;
+  p.gate_sb = gate_sb;
+  p.rows_per_batch = (int)rows_per_batch;
+  return gemm_dispatch(p, M, N, K, (hipStream_t)stream);
+}
+
+extern "C" int dsx_fp8_gemv_rowscale(const void* a, int64_t lda, const void* w, int64_t ldw,
+                                     const float* a_scale, const float* w_row_scale, const void* bias,
+                                     void* out, int64_t ldo, int64_t M, int64_t N, int64_t K,
+                                     void* stream) {
+  dsx::GemmArgs p;
+  const int rc = gemm_fill(p, a, lda, w, ldw, a_scale, nullptr, bias, out, ldo, M, N, K);
+  if (rc != DSX_OK || M == 0) return rc;
+  if (M > 8) return DSX_EBADSHAPE;
+  if (!w_row_scale) return DSX_ENULL;
+  p.w_row_scale = w_row_scale;
+  return gemm_dispatch(p, M, N, K, (hipStream_t)stream);
 }

@@ -5,9 +5,14 @@ Same inputs/outputs and state-dict names as ``FluxDiT.forward``
 (FluxJointTransformerBlock.forward :219-236, FluxSingleTransformerBlock.forward :308-321,
 FluxJointAttention.forward :161-194) are issued as a fixed sequence of libdsx kernels:
 
-  AdaLN-modulate (+ e4m3 emission) -> FP8 GEMM -> flash attention reading q/k/v straight out of
-  the packed qkv projection by stride, RMSNorm + RoPE fused, text-first joint sequence from two base
-  pointers (no chunk/concat copies) -> quantise -> FP8 GEMM -> gated residual -> ...
+  AdaLN-modulate (+ e4m3 emission) -> FP8 GEMM -> RMSNorm+RoPE in place -> flash attention reading
+  q/k/v straight out of the packed qkv projection by stride (text-first joint sequence from two base
+  pointers, no chunk/concat copies) -> quantise -> FP8 GEMM with the gated residual in its epilogue
+  -> AdaLN-modulate -> FP8 GEMM -> GELU (+ e4m3 emission) -> FP8 GEMM with gated residual.
+
+Every AdaLN projection consumes the same silu(conditioning) (transformer_helper.py:14,33;
+flux_dit.py:332), so all of them are stacked into one weight matrix at construction and evaluated
+by a single HBM-bound pass per step.
 
 All Linear layers run as per-token x per-tensor scaled e4m3 GEMMs (``scaled=True``) or with the
 reference's bare casts and unit scales (``scaled=False``, utils/fp8_linear.py:28-60).
@@ -40,15 +45,16 @@ class _Linear:
         self.b = None if bias is None else bias.to(torch.bfloat16).contiguous()
         self.n, self.k = self.w.shape
 
-    def __call__(self, a_q: torch.Tensor, a_s: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
-        return ops.fp8_gemm(a_q, self.w, a_s if self.s is not None else None, self.s, self.b, out=out)
+    def __call__(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
+        return ops.fp8_gemm(a_q, self.w, a_s if self.s is not None else None, self.s, self.b, out=out,
+                            resid=resid, gate=gate, rows_per_batch=rows_per_batch)
 
 
 class FluxDiTRunner:
     """Holds quantised weights of a Flux.1-dev-architecture DiT and runs one denoising step."""
 
-    def __init__(self, state_dict: Dict[str, torch.Tensor], num_double: int = 19, num_single: int = 38,
-                 scaled: bool = True, device="cuda:0", fuse_rope_in_attention: bool = False):
+    def __init__(self, state_dict, num_double: int = 19, num_single: int = 38, scaled: bool = True,
+                 device="cuda:0", fuse_rope_in_attention: bool = False):
         self.device = torch.device(device)
         self.scaled = scaled
         # True: RMSNorm/RoPE applied inside the attention kernel's tile loads; False: one in-place pre-pass
@@ -67,7 +73,28 @@ class FluxDiTRunner:
             elif key.endswith(".bias"):
                 self.lin[key[: -len(".bias")]].b = t.to(self.device, torch.bfloat16).contiguous()
         self.has_guidance = "guidance_embedder.timestep_embedder.0" in self.lin
-        self._rope_cache = {}
+        self._stack_modulation()
+
+    def _stack_modulation(self):
+        """One (N_total, 3072) e4m3 matrix holding every AdaLN projection, with a weight scale per row."""
+        names = []
+        for i in range(self.num_double):
+            names += [f"blocks.{i}.norm1_a.linear", f"blocks.{i}.norm1_b.linear"]
+        names += [f"single_blocks.{i}.norm.linear" for i in range(self.num_single)]
+        names.append("final_norm_out.linear")
+        self.mod_slices, off = {}, 0
+        ws, ss, bs = [], [], []
+        one = torch.ones((), dtype=torch.float32, device=self.device)
+        for n in names:
+            L = self.lin.pop(n)
+            self.mod_slices[n] = (off, off + L.n)
+            off += L.n
+            ws.append(L.w)
+            ss.append((L.s if L.s is not None else one).expand(L.n))
+            bs.append(L.b if L.b is not None else torch.zeros(L.n, dtype=torch.bfloat16, device=self.device))
+        self.mod_w = torch.cat(ws, dim=0)
+        self.mod_row_scale = torch.cat(ss).contiguous()
+        self.mod_bias = torch.cat(bs).contiguous()
 
     # ------------------------------------------------------------------ small helpers
     def _linear_bf16(self, x: torch.Tensor, name: str) -> torch.Tensor:
@@ -95,6 +122,12 @@ class FluxDiTRunner:
             ang = ids[..., a].unsqueeze(-1) * omega
             cols.append(torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1))
         return torch.cat(cols, dim=-2).float().contiguous()
+
+    def _modulations(self, cond: torch.Tensor) -> Dict[str, torch.Tensor]:
+        """linear(silu(cond)) of every AdaLN layer: one pass over the stacked weights."""
+        a_q, a_s = ops.quantize_fp8(torch.nn.functional.silu(cond), scaled=self.scaled)
+        out = ops.fp8_gemv_rowscale(a_q, self.mod_w, a_s, self.mod_row_scale, self.mod_bias)
+        return {n: out[:, lo:hi] for n, (lo, hi) in self.mod_slices.items()}
 
     def _modulate_q(self, x, scale, shift):
         """LayerNorm-modulate straight to the GEMM operand format."""
@@ -144,17 +177,17 @@ class FluxDiTRunner:
         return img, txt
 
     def _stream_tail(self, pre, s, x, attn_out, m):
-        """out-projection, gated residual, LN-modulate, MLP, gated residual of one stream (flux_dit.py:226-234)."""
+        """out-projection + gated residual, LN-modulate, MLP + gated residual of one stream (flux_dit.py:226-234)."""
         L = self.lin
         B, S, d = x.shape
+        x2 = x.reshape(B * S, d)
         q, sc = ops.quantize_fp8(attn_out, scaled=self.scaled)
-        proj = L[pre + f"attn.{s}_to_out"](q, sc).view(B, S, d)
-        x = ops.gated_residual(x, proj, m[2])
-        q, sc = self._modulate_q(x, m[4], m[3])
+        x2 = L[pre + f"attn.{s}_to_out"](q, sc, resid=x2, gate=m[2], rows_per_batch=S)
+        q, sc = self._modulate_q(x2.view(B, S, d), m[4], m[3])
         h = L[pre + f"ff_{s}.0"](q.view(-1, d), sc)
         q, sc = self._gelu_q(h)
-        h = L[pre + f"ff_{s}.2"](q, sc).view(B, S, d)
-        return ops.gated_residual(x, h, m[5])
+        x2 = L[pre + f"ff_{s}.2"](q, sc, resid=x2, gate=m[5], rows_per_batch=S)
+        return x2.view(B, S, d)
 
     def _single_block(self, i: int, x, mod, rope):
         """x (B,S,d); mod (B,3d) = shift, scale, gate (transformer_helper.py:34)."""
@@ -164,22 +197,26 @@ class FluxDiTRunner:
         shift, scale, gate = mod.chunk(3, dim=1)
         q, sc = self._modulate_q(x, scale, shift)
         h = L[pre + "to_qkv_mlp"](q.view(-1, d), sc)  # (B*S, 7d): [q | k | v | mlp]
-        cat = torch.empty((B * S, 5 * d), dtype=torch.bfloat16, device=x.device)
+        att = torch.empty((B, S, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=x.device)
         qkv = h.view(B, S, 7 * d)[:, :, : 3 * d].unflatten(2, (3 * HEADS, HEAD_DIM)).transpose(1, 2)
-        o = cat.view(B, S, 5 * d)[:, :, :d].unflatten(2, (HEADS, HEAD_DIM)).transpose(1, 2)
         nw = self.norm_w
         q_, k_, v_ = qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:]
         if self.fuse_rope_in_attention:
             ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
-                               eps=EPS, out=o)
+                               eps=EPS, out=att.transpose(1, 2))
         else:
             ops.rmsnorm_rope(q_, nw[pre + "norm_q_a"], rope, 0, EPS, out=q_)
             ops.rmsnorm_rope(k_, nw[pre + "norm_k_a"], rope, 0, EPS, out=k_)
-            ops.attention_bhsd(q_, k_, v_, out=o)
-        ops.gelu_tanh(h[:, 3 * d:], want_bf16=True, out=cat[:, d:])
-        q, sc = ops.quantize_fp8(cat, scaled=self.scaled)
-        proj = L[pre + "proj_out"](q, sc).view(B, S, d)
-        return ops.gated_residual(x, proj, gate)
+            ops.attention_bhsd(q_, k_, v_, out=att.transpose(1, 2))
+        # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
+        # parts and emits the e4m3 operand of proj_out with its per-token scale
+        if self.scaled:
+            q, sc = ops.concat_gelu_tanh(att.view(B * S, d), h[:, 3 * d:], want_fp8=True)
+        else:
+            q, sc = ops.quantize_fp8(ops.concat_gelu_tanh(att.view(B * S, d), h[:, 3 * d:], want_bf16=True,
+                                                          want_fp8=False), scaled=False)
+        out = L[pre + "proj_out"](q, sc, resid=x.reshape(B * S, d), gate=gate, rows_per_batch=S)
+        return out.view(B, S, d)
 
     # ------------------------------------------------------------------ step
     @torch.no_grad()
@@ -202,20 +239,16 @@ class FluxDiTRunner:
         x = hidden_states.to(bf).view(B, C, Hh // 2, 2, Ww // 2, 2).permute(0, 2, 4, 1, 3, 5)
         img = self._linear_bf16(x.reshape(B, (Hh // 2) * (Ww // 2), C * 4), "x_embedder")
 
-        # every AdaLN projection consumes the same silu(cond): quantise it once
-        sc_q, sc_s = ops.quantize_fp8(torch.nn.functional.silu(cond), scaled=self.scaled)
+        mods = self._modulations(cond)
         for i in range(self.num_double):
-            mod_a = self.lin[f"blocks.{i}.norm1_a.linear"](sc_q, sc_s)
-            mod_b = self.lin[f"blocks.{i}.norm1_b.linear"](sc_q, sc_s)
-            img, txt = self._joint_block(i, img, txt, mod_a, mod_b, rope)
+            img, txt = self._joint_block(i, img, txt, mods[f"blocks.{i}.norm1_a.linear"],
+                                         mods[f"blocks.{i}.norm1_b.linear"], rope)
         St = txt.shape[1]
         x = torch.cat([txt, img], dim=1)
         for i in range(self.num_single):
-            mod = self.lin[f"single_blocks.{i}.norm.linear"](sc_q, sc_s)
-            x = self._single_block(i, x, mod, rope)
+            x = self._single_block(i, x, mods[f"single_blocks.{i}.norm.linear"], rope)
         x = x[:, St:]
-        mod = self.lin["final_norm_out.linear"](sc_q, sc_s)
-        scale, shift = mod.chunk(2, dim=1)  # AdaLayerNormContinuous: scale first (flux_dit.py:333)
+        scale, shift = mods["final_norm_out.linear"].chunk(2, dim=1)  # AdaLayerNormContinuous: scale first (:333)
         q, s = self._modulate_q(x, scale, shift)
         out = self.lin["final_proj_out"](q.view(-1, HIDDEN), s).view(B, Hh // 2, Ww // 2, C, 2, 2)
         return out.permute(0, 3, 1, 4, 2, 5).reshape(B, C, Hh, Ww)

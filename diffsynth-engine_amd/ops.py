@@ -88,8 +88,12 @@ def quantize_weight_fp8(w: torch.Tensor, scaled: bool = True):
 
 def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor] = None,
              w_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3."""
+             out: Optional[torch.Tensor] = None, resid: Optional[torch.Tensor] = None,
+             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None) -> torch.Tensor:
+    """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3.
+
+    With ``resid`` (M,N) the gated residual is fused: out = resid + gate * that, gate (B,N) or None,
+    rows_per_batch = rows of a per batch entry (default: all M rows share gate row 0)."""
     _require_cuda(a_q, w_q)
     if a_q.dtype != FP8 or w_q.dtype != FP8:
         raise ValueError("fp8_gemm expects float8_e4m3fn operands")
@@ -111,9 +115,36 @@ def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tenso
         bias = bias.contiguous()
     if a_scale is not None:
         a_scale = a_scale.contiguous()
-    rc = _lib.load().dsx_fp8_gemm(_ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale), _ptr(w_scale),
-                                  _ptr(bias), _ptr(out), out.stride(0), M, N, K, _stream())
-    _lib.check(rc, "dsx_fp8_gemm")
+    if resid is None:
+        rc = _lib.load().dsx_fp8_gemm(_ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale),
+                                      _ptr(w_scale), _ptr(bias), _ptr(out), out.stride(0), M, N, K, _stream())
+        _lib.check(rc, "dsx_fp8_gemm")
+        return out
+    if resid.dtype != _BF16 or resid.shape != (M, N) or resid.stride(1) != 1:
+        raise ValueError("fp8_gemm: `resid` must be bf16 (M,N) with unit column stride")
+    gate_sb = 0
+    if gate is not None:
+        gate = gate.reshape(-1, N)
+        if gate.dtype != _BF16 or gate.stride(1) != 1:
+            gate = gate.to(_BF16).contiguous()
+        gate_sb = gate.stride(0) if gate.shape[0] > 1 else 0
+    rc = _lib.load().dsx_fp8_gemm_gated_residual(
+        _ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale), _ptr(w_scale), _ptr(bias), _ptr(resid),
+        resid.stride(0), _ptr(gate), gate_sb, rows_per_batch or M, _ptr(out), out.stride(0), M, N, K, _stream())
+    _lib.check(rc, "dsx_fp8_gemm_gated_residual")
+    return out
+
+
+def fp8_gemv_rowscale(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor],
+                      w_row_scale: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Small-M (<= 8) product against a stack of Linear weights with one fp32 weight scale per output row."""
+    _require_cuda(a_q, w_q)
+    M, K = a_q.shape
+    N = w_q.shape[0]
+    out = torch.empty((M, N), dtype=_BF16, device=a_q.device)
+    rc = _lib.load().dsx_fp8_gemv_rowscale(_ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale),
+                                           _ptr(w_row_scale), _ptr(bias), _ptr(out), N, M, N, K, _stream())
+    _lib.check(rc, "dsx_fp8_gemv_rowscale")
     return out
 
 
@@ -312,6 +343,26 @@ def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, o
         res.append(out if out is not None else y.view(shp))
     if want_fp8:
         res += [q.view(shp), qs]
+    return res[0] if len(res) == 1 else tuple(res)
+
+
+def concat_gelu_tanh(prefix: torch.Tensor, x: torch.Tensor, want_bf16: bool = False, want_fp8: bool = True):
+    """[prefix | gelu_tanh(x)] along the last dim for 2-D (rows, D) views; bf16 and/or per-token e4m3 output."""
+    _require_cuda(prefix, x)
+    if prefix.dtype != _BF16 or x.dtype != _BF16 or prefix.dim() != 2 or x.dim() != 2:
+        raise ValueError("concat_gelu_tanh expects 2-D bf16 tensors")
+    p2, ldp = _rows_2d(prefix)
+    x2, ldx = _rows_2d(x)
+    rows, Dp = p2.shape
+    D = x2.shape[1]
+    Dt = Dp + D
+    y = torch.empty((rows, Dt), dtype=_BF16, device=x.device) if want_bf16 else None
+    q = torch.empty((rows, Dt), dtype=FP8, device=x.device) if want_fp8 else None
+    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
+    rc = _lib.load().dsx_concat_gelu_tanh(_ptr(p2), ldp, Dp, _ptr(x2), ldx, _ptr(y), Dt, _ptr(q), Dt, _ptr(qs), rows,
+                                          D, _stream())
+    _lib.check(rc, "dsx_concat_gelu_tanh")
+    res = ([y] if want_bf16 else []) + ([q, qs] if want_fp8 else [])
     return res[0] if len(res) == 1 else tuple(res)
 
 

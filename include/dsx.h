@@ -88,6 +88,30 @@ int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t ldw, const f
                  int64_t N, int64_t K, void* stream);
 
 /*
+ * dsx_fp8_gemm with the gated residual of the DiT blocks fused into its epilogue:
+ *   proj = bf16( acc * a_scale[m] * w_scale + bias[n] );   out[m,n] = bf16( resid[m,n] + bf16(gate[b,n] * proj) )
+ * (gate == NULL: out = bf16(resid + proj)); b = m / rows_per_batch, gate row stride gate_sb.
+ * Replaces the `x + gate * linear(...)` pairs at models/flux/flux_dit.py:227,229,232,234,318-319 and
+ * models/wan/wan_dit.py:189,190,192 without the separate read-modify-write pass.
+ * `out` may be `resid` itself.
+ */
+int dsx_fp8_gemm_gated_residual(const void* a, int64_t lda, const void* w, int64_t ldw,
+                                const float* a_scale, const float* w_scale, const void* bias,
+                                const void* resid, int64_t ldr, const void* gate, int64_t gate_sb,
+                                int64_t rows_per_batch, void* out, int64_t ldo, int64_t M, int64_t N,
+                                int64_t K, void* stream);
+
+/*
+ * Small-M (M <= 8) form of dsx_fp8_gemm with one weight scale PER OUTPUT ROW (w_row_scale[n]), so that
+ * several Linear layers that consume the same activation can be stacked into one (N_total, K) weight
+ * and evaluated by one HBM-bound pass.  Used for the AdaLN projections, which all consume
+ * silu(conditioning) (models/basic/transformer_helper.py:14,33; models/flux/flux_dit.py:332).
+ */
+int dsx_fp8_gemv_rowscale(const void* a, int64_t lda, const void* w, int64_t ldw, const float* a_scale,
+                          const float* w_row_scale, const void* bias, void* out, int64_t ldo, int64_t M,
+                          int64_t N, int64_t K, void* stream);
+
+/*
  * Flash attention, head dim 128, bf16 in/out, fp32 online softmax, non-causal, no mask.
  * Replaces `_attn_func(q, k, v)` = F.scaled_dot_product_attention in
  * diffsynth_engine/models/flux/flux_dit.py:21,182,267,303 and `attention()` in
@@ -170,6 +194,16 @@ int dsx_gated_residual(const void* x, int64_t ldx, const void* y, int64_t ldy, c
  */
 int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
                   float* q_scale, int64_t rows, int64_t D, void* stream);
+
+/*
+ * Concatenating tanh-GELU: output row = [ prefix (Dp, copied) | gelu_tanh(x) (D) ], emitted as bf16
+ * (ldy) and/or per-token-scaled e4m3 (ldq, q_scale) like dsx_gelu_tanh.  Replaces
+ * `torch.cat([attn_output, F.gelu(mlp_hidden_states, approximate="tanh")], dim=2)` of the
+ * single-stream block (models/flux/flux_dit.py:315-317).  Dp % 8 == 0, D % 8 == 0, Dp + D <= 16384.
+ */
+int dsx_concat_gelu_tanh(const void* prefix, int64_t ldp, int64_t Dp, const void* x, int64_t ldx, void* y,
+                         int64_t ldy, void* q, int64_t ldq, float* q_scale, int64_t rows, int64_t D,
+                         void* stream);
 
 /*
  * Flow-match Euler update: out = cast(float(latents) + float(v) * dt), element-wise, bf16 or fp32

@@ -126,3 +126,39 @@ def test_flow_match_euler_step(dev):
         want = (a.to(torch.float32) + b * dt).to(dtype)
         got = ops.flow_match_euler_step(a.to(dev), b.to(dev), dt.item()).cpu()
         assert torch.equal(got, want)
+
+
+def test_concat_gelu_builds_single_block_operand(dev):
+    """[attention | gelu(mlp)] emitted as the per-token-scaled e4m3 operand of proj_out (flux_dit.py:315-317)."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(2)
+    rows, d = 21, 3072
+    att = torch.randn(rows, d, generator=g).bfloat16()
+    h = (torch.randn(rows, 7 * d, generator=g) * 2).bfloat16()
+    want = torch.cat([att, O.gelu_tanh(h[:, 3 * d:])], dim=1)
+    y, q, qs = ops.concat_gelu_tanh(att.to(dev), h.to(dev)[:, 3 * d:], want_bf16=True, want_fp8=True)
+    assert torch.equal(y.cpu()[:, :d], att)
+    frac, rel = _ulp_report(y.cpu(), want)
+    assert frac < 1e-3 and rel <= 2 ** -7, (frac, rel)
+    wq, ws = ofp8.quantize_rowwise(y.cpu(), scaled=True)
+    assert torch.equal(qs.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8), wq.view(torch.uint8))
+
+
+def test_adaln_wave_per_row_path_many_rows(dev):
+    """Rows >= 1024 take the one-wavefront-per-row kernel: same results, ragged row count."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(8)
+    for D in (3072, 5120):
+        x = torch.randn(1, 1027, D, generator=g).bfloat16()
+        mod = torch.randn(1, 2 * D, generator=g).bfloat16()
+        sc, sh = mod.chunk(2, dim=1)
+        want = O.layer_norm_modulate(x, sc[:, None], sh[:, None], 1e-6)
+        md = mod.to(dev)
+        scd, shd = md.chunk(2, dim=1)
+        y, q, qs = ops.adaln_modulate(x.to(dev), scd, shd, want_bf16=True, want_fp8=True)
+        frac, rel = _ulp_report(y.cpu(), want)
+        assert frac < 1e-3 and rel <= 2 ** -6, (D, frac, rel)
+        wq, ws = ofp8.quantize_rowwise(y.cpu().reshape(-1, D), scaled=True)
+        assert torch.equal(qs.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8).reshape(-1, D), wq.view(torch.uint8))

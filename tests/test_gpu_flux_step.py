@@ -81,14 +81,13 @@ def test_blocks_teacher_forced_against_oracle(dev):
     freqs = O.rope_table(ids, oflux.AXES_DIM, oflux.THETA)
     rope = ops.rope_table_from_freqs(freqs).to(dev)
     want_a, want_b = oflux.joint_block(P, 0, img, txt, cond, freqs)
-    sc_q, sc_s = ops.quantize_fp8(torch.nn.functional.silu(cond).to(dev), scaled=True)
-    mod_a = R.lin["blocks.0.norm1_a.linear"](sc_q, sc_s)
-    mod_b = R.lin["blocks.0.norm1_b.linear"](sc_q, sc_s)
-    got_a, got_b = R._joint_block(0, img.to(dev), txt.to(dev), mod_a, mod_b, rope)
+    mods = R._modulations(cond.to(dev))
+    got_a, got_b = R._joint_block(0, img.to(dev), txt.to(dev), mods["blocks.0.norm1_a.linear"],
+                                  mods["blocks.0.norm1_b.linear"], rope)
     assert _cos(got_a, want_a) >= 0.9995 and _cos(got_b, want_b) >= 0.9995, (_cos(got_a, want_a), _cos(got_b, want_b))
     x = torch.cat([txt, img], dim=1)
     want = oflux.single_block(P, 0, x, cond, freqs)
-    got = R._single_block(0, x.to(dev), R.lin["single_blocks.0.norm.linear"](sc_q, sc_s), rope)
+    got = R._single_block(0, x.to(dev), mods["single_blocks.0.norm.linear"], rope)
     assert _cos(got, want) >= 0.9995, _cos(got, want)
 
 

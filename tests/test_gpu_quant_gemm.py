@@ -127,3 +127,57 @@ def test_gemm_rejects_bad_arguments(dev):
         ops.fp8_gemm(a, w)  # K % 16 != 0
     with pytest.raises(ValueError):
         ops.fp8_gemm(a.bfloat16(), w)
+
+
+@pytest.mark.parametrize("M,N,K,B", [(512, 768, 256, 2), (300, 3072, 1024, 1), (260, 200, 128, 2), (96, 100, 64, 1)])
+def test_fp8_gemm_fused_gated_residual(dev, M, N, K, B):
+    """out = resid + gate * linear(x) with the gate row chosen per batch entry (flux_dit.py:227,318-319):
+    the fused epilogue must reproduce the three bf16 roundings of the separate ops."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(M + N)
+    w = torch.randn(N, K, generator=g) * 0.02
+    x = torch.randn(M, K, generator=g).bfloat16()
+    b = torch.randn(N, generator=g).bfloat16()
+    resid = torch.randn(M, N, generator=g).bfloat16()
+    gate = torch.randn(B, N, generator=g).bfloat16()
+    wq, ws = ofp8.quantize_weight(w)
+    xq, xs = ofp8.quantize_rowwise(x)
+    proj = ofp8.scaled_linear(xq, xs, wq, ws, b)
+    rows = M // B
+    assert rows * B == M
+    want = resid + gate.repeat_interleave(rows, dim=0) * proj
+    args = (xq.to(dev), wq.to(dev), xs.to(dev), ws.to(dev), b.to(dev))
+    got = ops.fp8_gemm(*args, resid=resid.to(dev), gate=gate.to(dev), rows_per_batch=rows).cpu()
+    plain = ops.fp8_gemm(*args).cpu()
+    # identical to applying the oracle's residual arithmetic to the kernel's own projection ...
+    assert torch.equal(got, resid + gate.repeat_interleave(rows, dim=0) * plain)
+    # ... and within accumulation-order noise of the all-oracle result
+    assert (got.float() - want.float()).abs().max().item() <= 2e-2 * want.float().abs().max().item()
+    want_nogate = resid + plain
+    assert torch.equal(ops.fp8_gemm(*args, resid=resid.to(dev)).cpu(), want_nogate)
+    # in place on the residual buffer
+    r_dev = resid.to(dev)
+    ops.fp8_gemm(*args, resid=r_dev, gate=gate.to(dev), rows_per_batch=rows, out=r_dev)
+    assert torch.equal(r_dev.cpu(), got)
+
+
+def test_fp8_gemv_rowscale_stacks_linears(dev):
+    """Three Linear layers with their own per-tensor scales evaluated as one stacked product == three products."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    K = 3072
+    x = torch.randn(2, K, generator=g).bfloat16()
+    xq, xs = ofp8.quantize_rowwise(x)
+    ws, ss, bs, want = [], [], [], []
+    for n, std in ((515, 0.02), (64, 0.5), (1030, 0.003)):
+        w = torch.randn(n, K, generator=g) * std
+        b = torch.randn(n, generator=g).bfloat16()
+        wq, s = ofp8.quantize_weight(w)
+        ws.append(wq); ss.append(s.expand(n)); bs.append(b)
+        want.append(ofp8.scaled_linear(xq, xs, wq, s, b))
+    got = ops.fp8_gemv_rowscale(xq.to(dev), torch.cat(ws).to(dev), xs.to(dev), torch.cat(ss).contiguous().to(dev),
+                                torch.cat(bs).to(dev)).cpu()
+    want = torch.cat(want, dim=1)
+    assert (got.float() - want.float()).abs().max().item() <= 1e-2 * want.float().abs().max().item()
