@@ -171,6 +171,63 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
                      red);
 }
 
+// RMSNorm over the whole row followed by an optional per-head RoPE (head dim 128, pairs (2i, 2i+1)):
+//   y = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ),  then  (c y0 - s y1, s y0 + c y1) -> bf16.
+// The row is a token's full model dim (Wan normalises q and k over all heads at once).
+template <int NCH, int TPR>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const uint16_t* __restrict__ x, int64_t ldx,
+                                                           const uint16_t* __restrict__ w, float eps,
+                                                           const float* __restrict__ rope, int64_t rope_sb,
+                                                           int64_t rows_per_batch, uint16_t* __restrict__ out,
+                                                           int64_t ldo, int64_t rows, int D) {
+  __shared__ float red[4];
+  const int t = threadIdx.x % TPR;
+  int64_t row = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
+  const bool live = row < rows;
+  if (!live) row = rows - 1;
+  const int nchunk = D >> 3;
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  float val[NCH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = t + i * TPR;
+    if (c < nchunk) {
+      unpack8(xr[c], val[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += val[i][j] * val[i][j];
+    }
+  }
+  const float rrms = rsqrtf(row_sum<TPR>(ss, red) / (float)D + eps);
+  if (!live) return;  // wave-uniform
+  const float* rp = rope ? rope + (row / rows_per_batch) * rope_sb + (row % rows_per_batch) * 128 : nullptr;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = t + i * TPR;
+    if (c < nchunk) {
+      float wv[8];
+      unpack8(reinterpret_cast<const u32x4*>(w)[c], wv);
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = round_bf16(round_bf16(val[i][j] * rrms) * wv[j]);
+      if (rp) {
+        const int off = (c * 8) & 127;  // offset inside the head: floats (cos, sin) of pairs off/2 .. off/2+3
+        const f32x4 t0 = *reinterpret_cast<const f32x4*>(rp + off);
+        const f32x4 t1 = *reinterpret_cast<const f32x4*>(rp + off + 4);
+        const float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float cc = cs[2 * k], sn = cs[2 * k + 1];
+          const float x0 = v[2 * k], x1 = v[2 * k + 1];
+          v[2 * k] = mul_add_unfused(cc, x0, -sn, x1);
+          v[2 * k + 1] = mul_add_unfused(sn, x0, cc, x1);
+        }
+      }
+      reinterpret_cast<u32x4*>(out + row * ldo)[c] = pack8(v);
+    }
+  }
+}
+
 // tanh-GELU of x, optionally preceded in the OUTPUT row by an unmodified prefix:
 // out row = [ prefix (Dp) | gelu(x) (D) ].  The prefix form is the single-stream block's
 // cat([attention, gelu(mlp)]) built directly in the operand format of proj_out.
@@ -366,5 +423,29 @@ extern "C" int dsx_flow_match_euler_step(const void* latents, const void* v, flo
     euler_step_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(latents, v, dt, out, n);
   else
     euler_step_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(latents, v, dt, out, n);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float eps, const float* rope,
+                                int64_t rope_sb, int64_t rows_per_batch, void* out, int64_t ldo, int64_t rows,
+                                int64_t D, void* stream) {
+  using namespace dsx;
+  if (!x || !w || !out) return DSX_ENULL;
+  if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || ldo < D || rows_per_batch <= 0 ||
+      (rope && (D & 127)))
+    return DSX_EBADSHAPE;
+  if ((ldx & 7) || (ldo & 7) || (rope_sb & 3) || misaligned16(x) || misaligned16(out) || misaligned16(w) ||
+      misaligned16(rope))
+    return DSX_EALIGN;
+  if (rows == 0) return DSX_OK;
+  hipStream_t st = (hipStream_t)stream;
+#define DSX_LAUNCH_RMS(NCH, TPR)                                                                           \
+  rmsnorm_rows_kernel<NCH, TPR><<<dim3((unsigned)((rows + 256 / TPR - 1) / (256 / TPR))), dim3(256), 0, st>>>( \
+      (const uint16_t*)x, ldx, (const uint16_t*)w, eps, rope, rope_sb, rows_per_batch, (uint16_t*)out, ldo,   \
+      rows, (int)D)
+  if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_RMS(6, 64);
+  else if (D <= 512 * 12 && rows >= 1024) DSX_LAUNCH_RMS(12, 64);
+  else DSX_LAUNCH_RMS(8, 256);
+#undef DSX_LAUNCH_RMS
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }

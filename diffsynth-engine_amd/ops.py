@@ -244,6 +244,36 @@ def rmsnorm_rope(x: torch.Tensor, norm_w: Optional[torch.Tensor], rope: Optional
     return out
 
 
+def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, rope: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Wan-style RMSNorm over the full last dim of (B,S,D) (or (rows,D)) bf16, optionally followed by RoPE on
+    every 128-wide head with the fp32 (B|1, S, 64, 2) (cos, sin) table."""
+    _require_cuda(x)
+    if x.dtype != _BF16:
+        raise ValueError("rmsnorm_rows expects bf16")
+    shp = x.shape
+    D = shp[-1]
+    x2, ldx = _rows_2d(x)
+    rows = x2.shape[0]
+    rows_per_batch = shp[-2] if x.dim() >= 2 else rows
+    rope_sb = 0
+    if rope is not None:
+        rope = rope.contiguous()
+        if rope.dtype != torch.float32 or rope.shape[-3:] != (rows_per_batch, 64, 2):
+            raise ValueError("rope table must be fp32 (B|1, S, 64, 2)")
+        rope_sb = rope.stride(0) if rope.dim() == 4 and rope.shape[0] > 1 else 0
+    if out is None:
+        out = torch.empty((rows, D), dtype=_BF16, device=x.device)
+        o2, ldo = out, D
+    else:
+        o2, ldo = _rows_2d(out)
+    w = weight.to(_BF16).contiguous()
+    rc = _lib.load().dsx_rmsnorm_rows(_ptr(x2), ldx, _ptr(w), eps, _ptr(rope), rope_sb, rows_per_batch, _ptr(o2), ldo,
+                                      rows, D, _stream())
+    _lib.check(rc, "dsx_rmsnorm_rows")
+    return out.view(shp)
+
+
 def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Optional[torch.Tensor],
                    eps: float = 1e-6, ln_weight=None, ln_bias=None, want_bf16: bool = True,
                    want_fp8: bool = False):

@@ -1,0 +1,150 @@
+"""Fused MI355X runner of the Wan2.1 DiT denoising step (text-to-video variant).
+
+Same inputs/outputs and state-dict names as ``WanDiT.forward``
+(diffsynth_engine/models/wan/wan_dit.py:319-351).  ``DiTBlock.forward`` (:185-193) is issued as:
+
+  AdaLN-modulate (+ e4m3) -> q/k/v FP8 GEMMs -> RMSNorm over the model dim + RoPE on q, k (one row kernel
+  each) -> flash attention over the (B,S,H*D) projections by stride -> quantise -> o GEMM with the gated
+  residual in its epilogue -> LayerNorm(affine) (+ e4m3) -> cross-attention against the text keys/values
+  (Lq != Lk) -> o GEMM with plain residual -> AdaLN-modulate -> FFN GEMM -> GELU (+ e4m3) -> FFN GEMM with
+  gated residual.
+
+The reference wires FP8 for Flux only (models/flux/flux_dit.py:404; pipelines/base.py:164-165 raises for the
+rest); here every Linear of the Wan DiT runs through the same scaled e4m3 GEMM as Flux.
+"""
+import math
+from typing import Dict
+
+import torch
+
+from . import ops
+from .flux_dit import _Linear
+
+
+class WanDiTRunner:
+    def __init__(self, state_dict, cfg: dict, scaled: bool = True, device="cuda:0"):
+        self.cfg = cfg
+        self.device = torch.device(device)
+        self.scaled = scaled
+        self.lin: Dict[str, _Linear] = {}
+        self.vec: Dict[str, torch.Tensor] = {}
+        d = cfg["dim"]
+        items = state_dict.items() if hasattr(state_dict, "items") else state_dict
+        for key, t in items:
+            if key == "patch_embedding.weight":  # Conv3d with kernel == stride == a Linear over each patch
+                self.lin["patch_embedding"] = _Linear(t.to(self.device).reshape(d, -1), None, scaled)
+            elif key.endswith(".weight") and t.dim() == 2:
+                self.lin[key[: -len(".weight")]] = _Linear(t.to(self.device), None, scaled)
+            elif key.endswith(".bias") and key[: -len(".bias")] in self.lin:
+                self.lin[key[: -len(".bias")]].b = t.to(self.device, torch.bfloat16).contiguous()
+            else:
+                self.vec[key] = t.to(self.device, torch.bfloat16).contiguous()
+
+    # ------------------------------------------------------------------ helpers
+    def _linear_bf16(self, x, name):
+        shp = x.shape
+        a_q, a_s = ops.quantize_fp8(x.reshape(-1, shp[-1]), scaled=self.scaled)
+        y = self.lin[name](a_q, a_s)
+        return y.view(*shp[:-1], y.shape[-1])
+
+    def _q(self, y):
+        return ops.quantize_fp8(y, scaled=self.scaled)
+
+    def _modulate_q(self, x, scale, shift, w=None, b=None):
+        if self.scaled:
+            return ops.adaln_modulate(x, scale, shift, self.cfg["eps"], ln_weight=w, ln_bias=b, want_bf16=False,
+                                      want_fp8=True)
+        return ops.quantize_fp8(ops.adaln_modulate(x, scale, shift, self.cfg["eps"], ln_weight=w, ln_bias=b),
+                                scaled=False)
+
+    def rope_table(self, f, h, w, theta=10000.0):
+        """(1, f*h*w, 64, 2) fp32 (cos, sin): head dim split (d - 2*(d//3), d//3, d//3) over (frame, row, col)
+        with float64 angles pos * theta^(-2j/dim_axis) (wan_dit.py:38-51,335-346)."""
+        hd = self.cfg["dim"] // self.cfg["num_heads"]
+        dev = self.device
+
+        def axis(dim, end):
+            fr = 1.0 / (theta ** (torch.arange(0, dim, 2, device=dev)[: dim // 2].double() / dim))
+            return torch.outer(torch.arange(end, device=dev).double(), fr)
+
+        af, ah, aw = axis(hd - 2 * (hd // 3), f), axis(hd // 3, h), axis(hd // 3, w)
+        ang = torch.cat([af.view(f, 1, 1, -1).expand(f, h, w, -1), ah.view(1, h, 1, -1).expand(f, h, w, -1),
+                         aw.view(1, 1, w, -1).expand(f, h, w, -1)], dim=-1).reshape(1, f * h * w, -1)
+        return torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).float().contiguous()
+
+    def _attention(self, q, k, v):
+        """(B,S,H*D) projections -> (B,S,H*D) attention output, head split/merge by strides (wan_dit.py:18-22)."""
+        H = self.cfg["num_heads"]
+        B, Sq, HD = q.shape
+        D = HD // H
+        sp = lambda t: t.view(t.shape[0], t.shape[1], H, D).transpose(1, 2)
+        out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=q.device)
+        ops.attention_bhsd(sp(q), sp(k), sp(v), out=out.transpose(1, 2))
+        return out.view(B * Sq, HD)
+
+    # ------------------------------------------------------------------ block
+    def block(self, i, x, context, t_mod, rope):
+        """DiTBlock.forward; x (B,S,d), context (B,Sc,d) already embedded, t_mod (B,6,d)."""
+        p = f"blocks.{i}."
+        L, V, eps = self.lin, self.vec, self.cfg["eps"]
+        B, S, d = x.shape
+        mod = (V[p + "modulation"] + t_mod).reshape(B, 6 * d)  # shift_msa, scale_msa, gate_msa, shift_mlp, ...
+        m = mod.chunk(6, dim=1)
+        x2 = x.reshape(B * S, d)
+        # self-attention
+        hq, hs = self._modulate_q(x, m[1], m[0])
+        hq = hq.view(B * S, d)
+        q = ops.rmsnorm_rows(L[p + "self_attn.q"](hq, hs).view(B, S, d), V[p + "self_attn.norm_q.weight"], eps, rope)
+        k = ops.rmsnorm_rows(L[p + "self_attn.k"](hq, hs).view(B, S, d), V[p + "self_attn.norm_k.weight"], eps, rope)
+        v = L[p + "self_attn.v"](hq, hs).view(B, S, d)
+        aq, asc = self._q(self._attention(q, k, v))
+        x2 = L[p + "self_attn.o"](aq, asc, resid=x2, gate=m[2], rows_per_batch=S)
+        # cross-attention (no gate on the residual)
+        hq, hs = self._modulate_q(x2.view(B, S, d), None, None, V[p + "norm3.weight"], V[p + "norm3.bias"])
+        q = ops.rmsnorm_rows(L[p + "cross_attn.q"](hq.view(B * S, d), hs).view(B, S, d),
+                             V[p + "cross_attn.norm_q.weight"], eps)
+        Sc = context.shape[1]
+        cq, cs = self._q(context.reshape(B * Sc, d))
+        k = ops.rmsnorm_rows(L[p + "cross_attn.k"](cq, cs).view(B, Sc, d), V[p + "cross_attn.norm_k.weight"], eps)
+        v = L[p + "cross_attn.v"](cq, cs).view(B, Sc, d)
+        aq, asc = self._q(self._attention(q, k, v))
+        x2 = L[p + "cross_attn.o"](aq, asc, resid=x2, gate=None, rows_per_batch=S)
+        # feed-forward
+        hq, hs = self._modulate_q(x2.view(B, S, d), m[4], m[3])
+        h = L[p + "ffn.0"](hq.view(B * S, d), hs)
+        if self.scaled:
+            gq, gs = ops.gelu_tanh(h, want_bf16=False, want_fp8=True)
+        else:
+            gq, gs = ops.quantize_fp8(ops.gelu_tanh(h), scaled=False)
+        x2 = L[p + "ffn.2"](gq, gs, resid=x2, gate=m[5], rows_per_batch=S)
+        return x2.view(B, S, d)
+
+    # ------------------------------------------------------------------ step
+    @torch.no_grad()
+    def forward(self, x, context, timestep):
+        cfg = self.cfg
+        d = cfg["dim"]
+        pf, ph, pw = cfg["patch_size"]
+        bf = torch.bfloat16
+        half = cfg["freq_dim"] // 2
+        ang = torch.outer(timestep.to(torch.float64),
+                          torch.pow(10000, -torch.arange(half, dtype=torch.float64, device=self.device).div(half)))
+        emb = torch.cat([torch.cos(ang), torch.sin(ang)], dim=1).to(bf)
+        t = self._linear_bf16(torch.nn.functional.silu(self._linear_bf16(emb, "time_embedding.0")), "time_embedding.2")
+        t_mod = self._linear_bf16(torch.nn.functional.silu(t), "time_projection.1").unflatten(1, (6, d))
+        ctx = ops.gelu_tanh(self._linear_bf16(context.to(bf), "text_embedding.0"))
+        ctx = self._linear_bf16(ctx, "text_embedding.2")
+        B, C, Fr, Hh, Ww = x.shape
+        f, h, w = Fr // pf, Hh // ph, Ww // pw
+        patches = x.to(bf).view(B, C, f, pf, h, ph, w, pw).permute(0, 2, 4, 6, 1, 3, 5, 7)
+        hs = self._linear_bf16(patches.reshape(B, f * h * w, C * pf * ph * pw), "patch_embedding")
+        rope = self.rope_table(f, h, w)
+        for i in range(cfg["num_layers"]):
+            hs = self.block(i, hs, ctx, t_mod, rope)
+        shift, scale = (self.vec["head.modulation"] + t).chunk(2, dim=1)  # Head.forward (wan_dit.py:234-237)
+        hq, hsc = self._modulate_q(hs, scale.reshape(B, d), shift.reshape(B, d))
+        out = self.lin["head.head"](hq.view(-1, d), hsc)
+        c = cfg["out_dim"]
+        return out.view(B, f, h, w, pf, ph, pw, c).permute(0, 7, 1, 4, 2, 5, 3, 6).reshape(B, c, f * pf, h * ph, w * pw)
+
+    __call__ = forward

@@ -163,6 +163,17 @@ int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss, co
                      int64_t seq, void* stream);
 
 /*
+ * RMSNorm over whole rows followed by an optional per-head RoPE (head dim 128):
+ *   y = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), then pairs (2i,2i+1) of every 128-wide head are rotated by
+ *   the (cos, sin) of table row (row % rows_per_batch) [+ rope_sb per batch entry] and rounded to bf16.
+ * Replaces Wan's RMSNorm.forward over the full model dim (models/wan/wan_dit.py:61-78,98-99,142-143) and
+ * rope_apply (wan_dit.py:54-58; the reference multiplies in complex128, this kernel in fp32).
+ * x, out: (rows, D) bf16; w: (D,) bf16; rope: fp32 (pos, 64, 2) or NULL.  D % 8 == 0 (128 with rope), D <= 16384.
+ */
+int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float eps, const float* rope, int64_t rope_sb,
+                     int64_t rows_per_batch, void* out, int64_t ldo, int64_t rows, int64_t D, void* stream);
+
+/*
  * AdaLN modulate: y = LayerNorm(x; eps, no affine) * (1 + scale) + shift, one row per token.
  * Replaces `self.norm(x) * (1 + scale) + shift` in models/basic/transformer_helper.py:17,21,35,
  * models/flux/flux_dit.py:228,233,334 and `modulate(norm(x), shift, scale)` in

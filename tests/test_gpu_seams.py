@@ -1,0 +1,87 @@
+"""GPU tests of the two drop-in seams as a reference user would reach them: the F.linear patch on real
+nn.Modules (utils/fp8_linear.py) and the attention callables installed into module globals."""
+import types
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from oracle import dit_ops as O
+from oracle import fp8 as ofp8
+
+pytestmark = pytest.mark.gpu
+
+
+class _Mlp(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.net = nn.Sequential(nn.Linear(256, 512), nn.GELU(approximate="tanh"), nn.Linear(512, 128, bias=False))
+
+    def forward(self, x):
+        return self.net(x)
+
+
+@pytest.mark.parametrize("scaled", [True, False])
+def test_enable_fp8_linear_and_fp8_inference_on_a_module(dev, scaled):
+    """enable_fp8_linear casts every floating nn.Linear weight in place and sets the flag FluxDiT.forward reads
+    (fp8_linear.py:7-17, flux_dit.py:404); under fp8_inference every nn.Linear.forward reaches the patched
+    F.linear (2-D and >2-D inputs, with and without bias)."""
+    from diffsynth_engine_amd import enable_fp8_linear, fp8_inference
+
+    torch.manual_seed(0)
+    m = _Mlp().to(torch.bfloat16)
+    ref_w = [m.net[0].weight.detach().clone(), m.net[2].weight.detach().clone()]
+    ref_b = m.net[0].bias.detach().clone()
+    m = m.to(dev)
+    enable_fp8_linear(m, scaled=scaled)
+    assert m.fp8_linear_enabled is True
+    assert m.net[0].weight.dtype == torch.float8_e4m3fn and m.net[0].bias.dtype == torch.bfloat16
+    assert hasattr(m.net[0].weight, "_dsx_scale") == scaled
+    x = torch.randn(3, 20, 256, generator=torch.Generator().manual_seed(1)).bfloat16()
+    orig = F.linear
+    with fp8_inference(getattr(m, "fp8_linear_enabled", False)):
+        y3 = m(x.to(dev))
+        y2 = m(x[0].to(dev))
+    assert F.linear is orig
+    # oracle: the same two linears through the reference arithmetic
+    wq0, ws0 = ofp8.quantize_weight(ref_w[0], scaled)
+    wq1, ws1 = ofp8.quantize_weight(ref_w[1], scaled)
+    h = O.gelu_tanh(ofp8.fp8_linear(x, wq0, ws0, ref_b))
+    want = ofp8.fp8_linear(h, wq1, ws1, None)
+    assert y3.shape == (3, 20, 128) and y2.shape == (20, 128) and y3.dtype == torch.bfloat16
+    cos = F.cosine_similarity(y3.cpu().float().flatten(), want.float().flatten(), dim=0).item()
+    assert cos >= 0.9995, cos
+    assert torch.equal(y2.cpu(), y3[0].cpu())
+    # weights quantised by the kernel are bit-identical to the oracle's
+    assert torch.equal(m.net[0].weight.data.cpu().view(torch.uint8), wq0.view(torch.uint8))
+
+
+def test_flux_seam_called_the_way_flux_joint_attention_calls_it(dev):
+    """_attn_func(q, k, v) positional, (B,H,S,D) non-contiguous views in, `.transpose(1,2).reshape` and `.to(dtype)`
+    applied to the result (flux_dit.py:182-184)."""
+    from diffsynth_engine_amd import set_attn_implementation
+
+    fake_flux_dit = types.SimpleNamespace(_attn_func=F.scaled_dot_product_attention)
+    set_attn_implementation("mi355x", flux_dit_module=fake_flux_dit)
+    B, S, H = 2, 200, 4
+    qkv = torch.randn(B, S, 3 * H * 128, generator=torch.Generator().manual_seed(2)).bfloat16()
+    qd, kd, vd = qkv.to(dev).view(B, S, 3 * H, 128).transpose(1, 2).chunk(3, dim=1)
+    hs = fake_flux_dit._attn_func(qd, kd, vd)
+    hs = hs.transpose(1, 2).reshape(B, -1, H * 128).to(qd.dtype)
+    q, k, v = qkv.view(B, S, 3 * H, 128).transpose(1, 2).chunk(3, dim=1)
+    want = O.sdpa(q.float(), k.float(), v.float()).transpose(1, 2).reshape(B, S, H * 128)
+    assert ((hs.cpu().float() - want).abs().max() / want.abs().max()).item() <= 2e-2
+    set_attn_implementation("sdpa", flux_dit_module=fake_flux_dit)
+    assert fake_flux_dit._attn_func is F.scaled_dot_product_attention
+
+
+def test_fp32_inputs_keep_their_dtype(dev):
+    """The reference runs CLIP/T5 in other dtypes through the same callables; outputs come back in the input dtype."""
+    from diffsynth_engine_amd import mi355x_attention
+
+    q = torch.randn(1, 2, 64, 128, generator=torch.Generator().manual_seed(3))
+    out = mi355x_attention(q.to(dev), q.to(dev), q.to(dev))
+    assert out.dtype == torch.float32
+    want = O.sdpa(q, q, q)
+    assert ((out.cpu() - want).abs().max() / want.abs().max()).item() <= 2e-2
