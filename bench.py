@@ -238,6 +238,13 @@ def cpu_baseline(num_double, num_single):
                       "extrapolated x%d + x%d (embedders and final layer excluded)" % (t1 - t0, t2 - t1, num_double, num_single)}
 
 
+# L2-miss bytes per fp8_gemm_kernel launch, averaged over the 230 launches of one 19+38 step:
+# rocprofv3 --pmc FETCH_SIZE (259.0 MB) plus --pmc WRITE_SIZE (59.8 MB), each scaled by what the same
+# counter reads for the 256 MiB copy of --calibrate-copy (FETCH_SIZE counts half the copied bytes,
+# WRITE_SIZE all of them); profiles/flux_step_hbm_traffic_pmc.txt holds the per-shape figures.
+GEMM_TRAFFIC_BYTES = 318.8e6
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -247,6 +254,9 @@ def main():
     ap.add_argument("--single", type=int, default=38)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy, the known-size dispatch that FETCH_SIZE / "
+                         "WRITE_SIZE counter runs are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one MI355X; this build has no multi-GPU path (--gpus must be 1)")
@@ -275,6 +285,12 @@ def main():
         guidance=torch.tensor([3.5], device=dev),
         text_ids=torch.zeros(1, N_TXT, 3, device=dev),
     )
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         out = runner(**inp)
     torch.cuda.synchronize()
@@ -309,7 +325,8 @@ def main():
                                "random init N(0,0.02), e4m3 weights (per-tensor scale), per-token activation scale"
                                % (args.double, args.single)},
         "roofline": {"bound": "mfma", "achieved": round(achieved / 1e12, 1), "peak": PEAK_FP8 / 1e12,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8, 4),
+                     "traffic": GEMM_TRAFFIC_BYTES if (args.double, args.single) == (19, 38) else None,
                      "kernel": "fp8_gemm_kernel", "launches": n_gemm,
                      "avg_launch_us": round(gemm_secs / max(n_gemm, 1) * 1e6, 1)},
         "step_roofline": {"algorithmic_tflop": round((gemm_fl + attn_fl) / 1e12, 2),

@@ -249,13 +249,8 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   for (int i = 0; i < 4; ++i) {
     const int row = (wave * 4 + i) * 16 + ld_r;
     const int c = ld_p ^ ((row >> 2) & 3);
-#ifdef DSX_EXPERIMENT_SAMETILE
-    w_src[i] = p.w + (int64_t)min(row, p.N - 1) * p.ldw + c * 16;
-    a_src[i] = p.a + (int64_t)min(row, p.M - 1) * p.lda + c * 16;
-#else
     w_src[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.ldw + c * 16;
     a_src[i] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.lda + c * 16;
-#endif
   }
   const int nk = p.K / SK;
   auto issue_load = [&](int kt, int stage, int idx) {
