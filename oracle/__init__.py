@@ -24,9 +24,18 @@ How each function is pinned (tests/test_oracle_*.py):
   sampler.*                               pinned against the reference's own golden files
                                           tests/data/expect/algorithm/{flow_match_euler_i10,
                                           recifited_flow_20steps_flux}.safetensors (copied as fixtures)
-  flux.* / wan.* block and model wiring   PARITY UNPINNED by any reference-held vector: the only
-                                          reference fixture on this path (tests/data/expect/flux/flux_dit.safetensors)
-                                          needs the 12B-parameter Flux.1-dev checkpoint.  Pinned only by
-                                          structural invariants (zero gates => identity, text rows see no
-                                          rotation, chunk orders checked against hand-built cases).
+  flux.ada_layer_norm6 / ada_layer_norm3 / rope_table / rms_norm / timestep_embedding, fp8.fp8_linear
+                                          pinned against vectors written by the reference's own leaf modules
+                                          (models/basic/transformer_helper.py, models/basic/timestep.py,
+                                          utils/fp8_linear.py; tests/golden/make_leaf_module_fixtures.py)
+  flux.joint_block / single_block / ada_layer_norm_continuous / flux_dit_forward
+                                          pinned against vectors written by the reference's own
+                                          FluxJointTransformerBlock, FluxSingleTransformerBlock,
+                                          AdaLayerNormContinuous and FluxDiT.forward at reduced width
+                                          (tests/golden/make_flux_block_fixtures.py), plus structural invariants
+  wan.freqs_cis_3d / dit_block / wan_dit_forward
+                                          pinned against vectors written by the reference's own WanDiT at
+                                          reduced size (tests/golden/make_wan_fixtures.py)
+The reference's only fixture on this path (tests/data/expect/flux/flux_dit.safetensors) needs the
+12B-parameter Flux.1-dev checkpoint and is not usable offline; full-size real-weight parity is unpinned.
 """

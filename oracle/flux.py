@@ -2,8 +2,8 @@
 
 Restates diffsynth_engine/models/flux/flux_dit.py:126-335,392-461 as functions over a flat dict of
 parameters whose keys are the reference's state-dict names (``blocks.3.attn.a_to_qkv.weight`` ...).
-Wiring is PARITY UNPINNED by reference-held vectors (see oracle/__init__.py); it is pinned by
-structural invariants in tests/test_oracle_flux.py.
+Wiring is pinned by vectors the reference's own classes wrote at reduced width
+(tests/test_oracle_leaf_goldens.py) and by structural invariants (tests/test_oracle_flux.py).
 
 ``linear_mode``:
   "plain"       F.linear in the tensors' dtype (the reference without enable_fp8_linear)
@@ -27,11 +27,13 @@ EPS = 1e-6
 class Params:
     """Flat parameter dict plus, in the fp8 modes, a cache of quantised weights."""
 
-    def __init__(self, tensors, linear_mode="plain"):
+    def __init__(self, tensors, linear_mode="plain", heads=HEADS, head_dim=HEAD_DIM, axes_dim=AXES_DIM):
         assert linear_mode in ("plain", "fp8_ref", "fp8_scaled")
         self.t = tensors
         self.linear_mode = linear_mode
         self._q = {}
+        # geometry: Flux.1-dev's unless a test builds a reduced model (flux_dit.py:343,352-356)
+        self.heads, self.head_dim, self.axes_dim = heads, head_dim, tuple(axes_dim)
 
     def __getitem__(self, k):
         return self.t[k]
@@ -97,10 +99,10 @@ def init_params(num_double=19, num_single=38, dtype=torch.bfloat16, device="cpu"
     return t
 
 
-def _heads(x):
+def _heads(x, heads=HEADS, head_dim=HEAD_DIM):
     """(B,S,3*H*D) -> q,k,v each (B,H,S,D): view as (B,S,3H,D), transpose, chunk(3) (flux_dit.py:165-167)."""
     B, S, _ = x.shape
-    x = x.view(B, S, 3 * HEADS, HEAD_DIM).transpose(1, 2)
+    x = x.view(B, S, 3 * heads, head_dim).transpose(1, 2)
     return x.chunk(3, dim=1)
 
 
@@ -111,10 +113,10 @@ def _merge(x):
 
 def joint_attention(P, pre, a, b, freqs, attn=O.sdpa):
     """FluxJointAttention.forward (flux_dit.py:161-194); a = image stream, b = text stream, text first."""
-    q_a, k_a, v_a = _heads(P.linear(a, pre + "a_to_qkv"))
+    q_a, k_a, v_a = _heads(P.linear(a, pre + "a_to_qkv"), P.heads, P.head_dim)
     q_a = O.rms_norm(q_a, P[pre + "norm_q_a.weight"], EPS)
     k_a = O.rms_norm(k_a, P[pre + "norm_k_a.weight"], EPS)
-    q_b, k_b, v_b = _heads(P.linear(b, pre + "b_to_qkv"))
+    q_b, k_b, v_b = _heads(P.linear(b, pre + "b_to_qkv"), P.heads, P.head_dim)
     q_b = O.rms_norm(q_b, P[pre + "norm_q_b.weight"], EPS)
     k_b = O.rms_norm(k_b, P[pre + "norm_k_b.weight"], EPS)
     q = torch.cat([q_b, q_a], dim=2)
@@ -133,6 +135,20 @@ def ada_layer_norm6(P, name, x, emb):
     e = P.linear(F.silu(emb), name + ".linear").unsqueeze(1)
     shift_msa, scale_msa, gate_msa, shift_mlp, scale_mlp, gate_mlp = e.chunk(6, dim=2)
     return O.layer_norm_modulate(x, scale_msa, shift_msa, EPS), gate_msa, shift_mlp, scale_mlp, gate_mlp
+
+
+def ada_layer_norm3(P, name, x, emb):
+    """AdaLayerNormSingle.forward (transformer_helper.py:32-36): chunk order shift, scale, gate."""
+    e = P.linear(F.silu(emb), name + ".linear")
+    shift, scale, gate = e.chunk(3, dim=1)
+    return O.layer_norm_modulate(x, scale[:, None], shift[:, None], EPS), gate
+
+
+def ada_layer_norm_continuous(P, name, x, cond):
+    """AdaLayerNormContinuous.forward (flux_dit.py:331-335): chunk order scale, shift."""
+    e = P.linear(F.silu(cond), name + ".linear")
+    scale, shift = torch.chunk(e, 2, dim=1)
+    return O.layer_norm_modulate(x, scale[:, None], shift[:, None], EPS)
 
 
 def joint_block(P, i, a, b, temb, freqs, attn=O.sdpa):
@@ -158,12 +174,11 @@ def single_block(P, i, x, temb, freqs, attn=O.sdpa):
     """FluxSingleTransformerBlock.forward + process_attention (flux_dit.py:294-321);
     AdaLayerNormSingle chunk order shift, scale, gate (transformer_helper.py:32-36)."""
     pre = f"single_blocks.{i}."
-    e = P.linear(F.silu(temb), pre + "norm.linear")
-    shift, scale, gate = e.chunk(3, dim=1)
-    n = O.layer_norm_modulate(x, scale[:, None], shift[:, None], EPS)
+    n, gate = ada_layer_norm3(P, pre + "norm", x, temb)
     h = P.linear(n, pre + "to_qkv_mlp")
-    qkv, mlp = h[:, :, : 3 * HIDDEN], h[:, :, 3 * HIDDEN:]
-    q, k, v = _heads(qkv)
+    d = P.heads * P.head_dim
+    qkv, mlp = h[:, :, : 3 * d], h[:, :, 3 * d:]
+    q, k, v = _heads(qkv, P.heads, P.head_dim)
     q = O.rms_norm(q, P[pre + "norm_q_a.weight"], EPS)
     k = O.rms_norm(k, P[pre + "norm_k_a.weight"], EPS)
     q, k = O.apply_rope(q, freqs), O.apply_rope(k, freqs)
@@ -215,7 +230,7 @@ def flux_dit_forward(P, hidden_states, timestep, prompt_emb, pooled_prompt_emb, 
         cond = cond + timestep_mlp(P, "guidance_embedder", guidance * 1000, dtype)
     cond = cond + P.linear(F.silu(P.linear(pooled_prompt_emb, "pooled_text_embedder.0")), "pooled_text_embedder.2")
     txt = P.linear(prompt_emb, "context_embedder")
-    freqs = O.rope_table(torch.cat((text_ids, img_ids), dim=1), AXES_DIM, THETA)
+    freqs = O.rope_table(torch.cat((text_ids, img_ids), dim=1), P.axes_dim, THETA)
     height, width = hidden_states.shape[-2:]
     img = P.linear(patchify(hidden_states), "x_embedder")
     for i in range(num_double):
@@ -224,9 +239,6 @@ def flux_dit_forward(P, hidden_states, timestep, prompt_emb, pooled_prompt_emb, 
     for i in range(num_single):
         x = single_block(P, i, x, cond, freqs, attn)
     x = x[:, txt.shape[1]:]
-    # AdaLayerNormContinuous (flux_dit.py:331-335): chunk order scale, shift
-    e = P.linear(F.silu(cond), "final_norm_out.linear")
-    scale, shift = torch.chunk(e, 2, dim=1)
-    x = O.layer_norm_modulate(x, scale[:, None], shift[:, None], EPS)
+    x = ada_layer_norm_continuous(P, "final_norm_out", x, cond)
     x = P.linear(x, "final_proj_out")
     return unpatchify(x, height, width)

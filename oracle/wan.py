@@ -1,9 +1,9 @@
 """Wan2.1 DiT block and model forward — oracle (test infrastructure, see oracle/__init__.py).
 
 Restates diffsynth_engine/models/wan/wan_dit.py:18-351 (text-to-video variant, has_image_input=False) as
-functions over a flat parameter dict whose keys are the reference's state-dict names.  Wiring is PARITY
-UNPINNED by reference-held vectors (the reference has no WanDiT test); pinned by structural invariants in
-tests/test_oracle_wan.py.  ``linear_mode`` as in oracle/flux.py.
+functions over a flat parameter dict whose keys are the reference's state-dict names.  The reference has
+no WanDiT test; wiring is pinned by vectors its own WanDiT class wrote at reduced size
+(tests/test_oracle_leaf_goldens.py) and by structural invariants (tests/test_oracle_wan.py).  ``linear_mode`` as in oracle/flux.py.
 """
 import math
 
