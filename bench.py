@@ -89,13 +89,15 @@ def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
 
 
 class GemmTimer:
-    """Brackets every fp8_gemm launch with events on the launch stream (torch's current stream, which is the
-    stream handed to the C-ABI) and accumulates algorithmic flops for launches with M > 8."""
+    """Brackets every fp8_gemm launch (single, or two problems sharing one grid) with events on the launch
+    stream (torch's current stream, which is the stream handed to the C-ABI) and accumulates algorithmic
+    flops for launches with M > 8."""
 
     def __init__(self, torch, ops):
         self.torch, self.ops = torch, ops
         self.records = []
         self._orig = ops.fp8_gemm
+        self._orig_grouped = ops.fp8_gemm_grouped
 
     def __enter__(self):
         torch, orig, rec = self.torch, self._orig, self.records
@@ -111,11 +113,23 @@ class GemmTimer:
             rec.append((e0, e1, 2.0 * M * K * w_q.shape[0]))
             return out
 
+        orig_grouped = self._orig_grouped
+
+        def timed_grouped(problems):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = orig_grouped(problems)
+            e1.record()
+            rec.append((e0, e1, sum(2.0 * p["a_q"].shape[0] * p["a_q"].shape[1] * p["w_q"].shape[0] for p in problems)))
+            return out
+
         self.ops.fp8_gemm = timed
+        self.ops.fp8_gemm_grouped = timed_grouped
         return self
 
     def __exit__(self, *exc):
         self.ops.fp8_gemm = self._orig
+        self.ops.fp8_gemm_grouped = self._orig_grouped
 
     def summary(self):
         self.torch.cuda.synchronize()

@@ -47,6 +47,25 @@ class AttnParams(ctypes.Structure):
     ]
 
 
+class GemmProblem(ctypes.Structure):
+    """Mirror of ``dsx_gemm_problem``."""
+
+    _fields_ = [
+        ("a", c_void_p), ("lda", c_int64),
+        ("w", c_void_p), ("ldw", c_int64),
+        ("a_scale", c_void_p),
+        ("w_scale", c_void_p),
+        ("bias", c_void_p),
+        ("resid", c_void_p), ("ldr", c_int64),
+        ("gate", c_void_p), ("gate_sb", c_int64),
+        ("rows_per_batch", c_int64),
+        ("out", c_void_p), ("ldo", c_int64),
+        ("M", c_int64), ("N", c_int64), ("K", c_int64),
+    ]
+
+
+GEMM_GROUP_MAX = 4
+
 # name -> (restype, argtypes); every symbol include/dsx.h declares
 SIGNATURES = {
     "dsx_abi_version": (c_int, []),
@@ -60,6 +79,7 @@ SIGNATURES = {
     "dsx_fp8_gemm_gated_residual": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
                                             c_int64, c_int64, c_int64, c_void_p]),
+    "dsx_fp8_gemm_grouped": (c_int, [ctypes.POINTER(GemmProblem), c_int, c_void_p]),
     "dsx_fp8_gemv_rowscale": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "dsx_concat_gelu_tanh": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,

@@ -10,11 +10,13 @@
 // quad, so the per-token scale is a per-lane constant and the bf16 results leave as 8-byte stores.
 //
 // Main kernel: 256x256 output tile per workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
-// tiles (256 fp32 accumulators), K step 128 bytes, two LDS stages of 64 KiB filled by
-// global_load_lds_dwordx4 (HBM/L2 -> LDS without staging registers) one full K step ahead,
-// MFMA operand fragments double-buffered in registers so that LDS reads overlap the MFMAs.
-// LDS rows are 128 B (8 chunks of 16 B); chunk c of row r lives at chunk c ^ ((r/2)&7), which
-// makes 16 lanes reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
+// tiles (256 fp32 accumulators).  Operands reach LDS by global_load_lds_dwordx4 (HBM/L2 -> LDS
+// without staging registers) in 128-byte-wide units through a five-slot ring; MFMA operand
+// fragments are double-buffered in registers so that LDS reads overlap the MFMAs.  LDS rows are
+// 128 B (8 chunks of 16 B); chunk c of row r lives at chunk c ^ ((r/2)&7), which makes 16 lanes
+// reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
+// One launch can carry two independent problems (the image- and text-stream linears of a joint
+// block): their tiles share the grid, so the small problem runs on CUs the large one leaves idle.
 #include "common.h"
 
 namespace dsx {
@@ -46,14 +48,34 @@ struct GemmArgs {
   const float* w_row_scale;
 };
 
-__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn,
-                                            bool& valid) {
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of
-  // logical tile ids so that tiles sharing A rows / W rows meet in the same L2.
-  const int total = tiles_m * tiles_n;
+// Two problems in one grid: logical tiles [0, tiles of p[0]) belong to p[0], the rest to p[1].
+struct GemmPair {
+  GemmArgs p[2];
+  int total0;  // tiles of p[0]
+  int total;   // tiles of both
+};
+
+// Field-wise select (all operands are wave-uniform, so this is a run of scalar selects; indexing
+// the kernel argument dynamically would copy both structs to scratch memory).
+__device__ __forceinline__ GemmArgs pick(const GemmPair& q, bool second) {
+  GemmArgs r;
+#define DSX_PICK(f) r.f = second ? q.p[1].f : q.p[0].f
+  DSX_PICK(a); DSX_PICK(w); DSX_PICK(a_scale); DSX_PICK(w_scale); DSX_PICK(bias); DSX_PICK(out);
+  DSX_PICK(lda); DSX_PICK(ldw); DSX_PICK(ldo); DSX_PICK(M); DSX_PICK(N); DSX_PICK(K);
+  DSX_PICK(tiles_m); DSX_PICK(tiles_n); DSX_PICK(resid); DSX_PICK(gate); DSX_PICK(ldr); DSX_PICK(gate_sb);
+  DSX_PICK(rows_per_batch); DSX_PICK(w_row_scale);
+#undef DSX_PICK
+  return r;
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of logical tile
+// ids so that tiles sharing A rows / W rows meet in the same L2.
+__device__ __forceinline__ int logical_tile(int wg, int total) {
   const int per_xcd = (total + 7) >> 3;
-  const int L = (wg & 7) * per_xcd + (wg >> 3);
-  valid = L < total;
+  return (wg & 7) * per_xcd + (wg >> 3);
+}
+
+__device__ __forceinline__ void tile_of(int L, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int G = 4;
   const int span = G * tiles_n;
   const int group = L / span;
@@ -62,6 +84,14 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
   const int rem = L - group * span;
   tm = first_m + rem % gsz;
   tn = rem / gsz;
+}
+
+__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn,
+                                            bool& valid) {
+  const int total = tiles_m * tiles_n;
+  const int L = logical_tile(wg, total);
+  valid = L < total;
+  tile_of(L, tiles_m, tiles_n, tm, tn);
 }
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -209,28 +239,33 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
 }
 
 // ------------------------------------------------------------------------------------------
-// Main kernel: K % 128 == 0.  Five LDS stages of one 64-byte K slab each (W tile 256x64 + A tile
-// 256x64 = 32 KiB per stage, 160 KiB in all), filled by global_load_lds_dwordx4 four slabs ahead:
-// a slab needs ~0.5 us just to stream through the CU's vector memory path on top of the L2/HBM
-// latency, so a one-slab lead leaves the MFMAs waiting on memory.
+// Main kernel: K % 128 == 0.  Operands move HBM -> LDS in units of one operand x 128 bytes of K
+// (256 rows x 128 B = 32 KiB), so that every async load instruction (64 lanes x 16 B) fetches
+// eight whole 128-byte cache lines: with 64-byte rows each line would be requested twice, a step
+// apart, and the second request stalls the L1 behind the still-pending first one.  Five unit
+// slots (160 KiB) form a ring W0 A0 W1 A1 W2 | A2 W3 ...; one MFMA step consumes 64 bytes of K,
+// i.e. half of a W unit and half of an A unit.
 // ------------------------------------------------------------------------------------------
-constexpr int SK = 64;                        // K bytes per stage
-constexpr int NSTAGE = 5;
-constexpr int kSlabTile = 256 * SK;           // one operand, 16 KiB
-constexpr int kSlabBytes = 2 * kSlabTile;     // 32 KiB
+constexpr int SK = 64;                   // K bytes per MFMA step
+constexpr int UK = 128;                  // K bytes per unit row
+constexpr int NSLOT = 5;
+constexpr int kUnitBytes = 256 * UK;     // 32 KiB
 
-// 64-byte rows: 16-byte chunk c of row r lives at chunk c ^ ((r/4)&3); four rows span the 64 banks.
-__device__ __forceinline__ int slab_off(int row, int chunk) {
-  return row * SK + ((chunk ^ ((row >> 2) & 3)) << 4);
+// 128-byte rows: 16-byte chunk c of row r lives at chunk c ^ ((r/2)&7); two rows span the 64 banks.
+__device__ __forceinline__ int unit_off(int row, int chunk) {
+  return row * UK + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
 template <bool RESID>
-__global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
+__global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmPair q) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  int L = logical_tile(blockIdx.x, q.total);
+  if (L >= q.total) return;
+  const bool second = L >= q.total0;
+  if (second) L -= q.total0;
+  const GemmArgs p = pick(q, second);
   int tm, tn;
-  bool valid;
-  tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn, valid);
-  if (!valid) return;
+  tile_of(L, p.tiles_m, p.tiles_n, tm, tn);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -239,43 +274,47 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
   const int g = lane >> 5, li = lane & 31;
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // ---- async loads: one wave instruction fills 1 KiB of LDS = 16 rows x 64 B; lane l lands at
-  //      row l/4, physical chunk l%4, so it fetches logical chunk (l%4) ^ swz(row).
-  //      Per slab a wave issues 8 instructions: 4 for its 64 W rows, 4 for its 64 A rows.
-  const int ld_r = lane >> 2, ld_p = lane & 3;
-  const uint8_t* w_src[4];
-  const uint8_t* a_src[4];
+  // ---- async loads: one wave instruction fills 1 KiB of LDS = 8 rows x 128 B; lane l lands at
+  //      row l/8, physical chunk l%8, so it fetches logical chunk (l%8) ^ swz(row).
+  //      Per unit a wave issues 8 instructions for its 64 rows.
+  const int ld_r = lane >> 3, ld_p = lane & 7;
+  uint32_t w_off[8], a_off[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = (wave * 4 + i) * 16 + ld_r;
-    const int c = ld_p ^ ((row >> 2) & 3);
-    w_src[i] = p.w + (int64_t)min(n0 + row, p.N - 1) * p.ldw + c * 16;
-    a_src[i] = p.a + (int64_t)min(m0 + row, p.M - 1) * p.lda + c * 16;
+  for (int i = 0; i < 8; ++i) {
+    const int row = (wave * 8 + i) * 8 + ld_r;
+    const int c = ld_p ^ ((row >> 1) & 7);
+    w_off[i] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.ldw + c * 16;
+    a_off[i] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.lda + c * 16;
   }
-  const int nk = p.K / SK;
-  auto issue_load = [&](int kt, int stage, int idx) {
-    kt = min(kt, nk - 1);  // past the end: re-fetch the last slab into a stage nobody reads again
-    uint8_t* dst = smem + stage * kSlabBytes + (idx & 1) * kSlabTile + (wave * 4 + (idx >> 1)) * 1024;
-    const uint8_t* src = ((idx & 1) ? a_src[idx >> 1] : w_src[idx >> 1]) + (int64_t)kt * SK;
+  const uint8_t* w_base = p.w + (int64_t)n0 * p.ldw;
+  const uint8_t* a_base = p.a + (int64_t)m0 * p.lda;
+  const int nk = p.K / SK;       // MFMA steps, even
+  const int nu = nk / 2;         // units per operand
+  // unit (j, op): op 0 = W, 1 = A; ring slot (2j + op) % 5
+  auto issue_load = [&](int j, int op, int i) {
+    const int slot = (2 * j + op) % NSLOT;
+    j = min(j, nu - 1);  // past the end: re-fetch the last unit into a slot nobody reads again
+    uint8_t* dst = smem + slot * kUnitBytes + (wave * 8 + i) * 1024;
+    const uint8_t* src = (op ? a_base + a_off[i] : w_base + w_off[i]) + (int64_t)j * UK;
     __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
   };
 
-  // ---- fragments: 4 W tiles + 4 A tiles, two 16-byte halves each = 16 LDS reads per slab
+  // ---- fragments: 4 W tiles + 4 A tiles, two 16-byte halves each = 16 LDS reads per step
   const int w_row = wn * 128 + li;
   const int a_row = wm * 128 + li;
   struct Frags {
     i32x4 w[4][2];
     i32x4 a[4][2];
   };
-  auto read_frag = [&](Frags& f, int stage, int idx) {
-    const uint8_t* sW = smem + stage * kSlabBytes;
-    const uint8_t* sA = sW + kSlabTile;
+  auto read_frag = [&](Frags& f, int j, int par, int idx) {   // fragments of MFMA step 2j + par
+    const uint8_t* sW = smem + ((2 * j) % NSLOT) * kUnitBytes;
+    const uint8_t* sA = smem + ((2 * j + 1) % NSLOT) * kUnitBytes;
     const int t = idx >> 2, half = idx & 1, is_a = (idx >> 1) & 1;
-    const int c = g * 2 + half;
+    const int c = par * 4 + g * 2 + half;
     if (is_a)
-      f.a[t][half] = *reinterpret_cast<const i32x4*>(sA + slab_off(a_row + t * 32, c));
+      f.a[t][half] = *reinterpret_cast<const i32x4*>(sA + unit_off(a_row + t * 32, c));
     else
-      f.w[t][half] = *reinterpret_cast<const i32x4*>(sW + slab_off(w_row + t * 32, c));
+      f.w[t][half] = *reinterpret_cast<const i32x4*>(sW + unit_off(w_row + t * 32, c));
   };
 
   f32x16 acc[4][4];
@@ -295,36 +334,43 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmArgs p) {
     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fw, fa, acc[i][j], 0, 0, 0, 0, 0, 0);
   };
 
-  // One step: slab s is in registers (fc).  Behind the barrier slab s+1 is in LDS (only the 16
-  // newest async loads, slabs s+2 and s+3, may still be in flight) and stage (s+4)%5 = (s-1)%5 has
-  // been read for the last time by every wave.  16 MFMAs, each followed by one LDS read of slab
-  // s+1 and, for the first eight, one async load of slab s+4; sched_barrier pins that order.
-  auto step = [&](int s, const Frags& fc, Frags& fn) {
-    __builtin_amdgcn_s_waitcnt(0x4070);  // vmcnt(16) lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    const int st_next = (s + 1) % NSTAGE, st_load = (s + 4) % NSTAGE;
+  // Step s multiplies the fragments of step s (in registers, fc) while reading those of step s+1.
+  // Even step 2j: its reads stay inside units j, already known to have landed; no barrier.  It
+  //   issues the loads of W unit j+2 into the slot A unit j-1 left at the last barrier.
+  // Odd step 2j+1: its reads open units j+1, so first wait until only the 8 newest loads (W unit
+  //   j+2) are in flight, then the barrier; that barrier also says every wave has read W unit j
+  //   for the last time, whose slot takes the loads of A unit j+2.
+  // 16 MFMAs, each followed by one LDS read and, for the first eight, one async load;
+  // sched_barrier pins that order.
+  auto step = [&](int j, int par, const Frags& fc, Frags& fn) {   // MFMA step 2j + par; par is a literal
+    if (par) {
+      __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+    } else {
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    }
 #pragma unroll
     for (int idx = 0; idx < 16; ++idx) {
       mfma_one(fc, idx);
-      read_frag(fn, st_next, idx);
-      if (idx < 8) issue_load(s + 4, st_load, idx);
+      read_frag(fn, j + par, par ^ 1, idx);
+      if (idx < 8) issue_load(j + 2, par, idx);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
   Frags f0, f1;
 #pragma unroll
-  for (int s = 0; s < 4; ++s)
+  for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int idx = 0; idx < 8; ++idx) issue_load(s, s, idx);
-  __builtin_amdgcn_s_waitcnt(0x4f78);  // vmcnt(24): slab 0 has landed
+    for (int i = 0; i < 8; ++i) issue_load(u >> 1, u & 1, i);
+  __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16): W and A unit 0 have landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int idx = 0; idx < 16; ++idx) read_frag(f0, 0, idx);
+  for (int idx = 0; idx < 16; ++idx) read_frag(f0, 0, 0, idx);
 
-  for (int s = 0; s < nk; s += 2) {  // nk is even (K % 128 == 0)
-    step(s, f0, f1);
-    step(s + 1, f1, f0);
+  for (int j = 0; j < nu; ++j) {
+    step(j, 0, f0, f1);
+    step(j, 1, f1, f0);
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is reused
 
@@ -479,17 +525,8 @@ static int launch_gemv(const GemmArgs& p, hipStream_t st) {
 
 }  // namespace dsx
 
-static int gemm_dispatch(dsx::GemmArgs& p, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+static int gemm_set_attributes() {
   using namespace dsx;
-  if (M <= 8) {
-    p.tiles_m = p.tiles_n = 0;
-    return launch_gemv(p, st);
-  }
-  if (p.w_row_scale) return DSX_EBADSHAPE;
-  p.tiles_m = (int)((M + BM - 1) / BM);
-  p.tiles_n = (int)((N + BN - 1) / BN);
-  const int total = p.tiles_m * p.tiles_n;
-  const int grid = ((total + 7) / 8) * 8;
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)fp8_gemm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -501,17 +538,50 @@ static int gemm_dispatch(dsx::GemmArgs& p, int64_t M, int64_t N, int64_t K, hipS
       return DSX_ELAUNCH;
     attr_set = true;
   }
+  return DSX_OK;
+}
+
+// Fills the tile counts and says whether the problem can run on the main 256x256 kernel.
+static bool gemm_main_kernel_ok(dsx::GemmArgs& p) {
+  using namespace dsx;
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
   const bool vec_ok = ((p.ldo & 7) == 0) && ((p.N & 7) == 0) && (((uintptr_t)p.out & 15) == 0) &&
                       (!p.bias || ((uintptr_t)p.bias & 7) == 0) &&
                       (!p.resid || ((((uintptr_t)p.resid & 15) == 0) && ((p.ldr & 7) == 0) &&
                                     (((uintptr_t)p.gate & 15) == 0) && ((p.gate_sb & 7) == 0)));
-  if ((K % 128) == 0 && vec_ok) {
-    if (p.resid)
-      fp8_gemm_kernel<true><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(p);
-    else
-      fp8_gemm_kernel<false><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(p);
-  } else
-    fp8_gemm_ragged_k_kernel<<<dim3((unsigned)grid), dim3(256), kStageBytes, st>>>(p);
+  return p.M > 8 && !p.w_row_scale && (p.K % 128) == 0 && vec_ok;
+}
+
+// One launch of the main kernel over one or two problems (both with or both without a residual).
+static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStream_t st) {
+  using namespace dsx;
+  GemmPair q;
+  q.p[0] = p0;
+  q.p[1] = p1 ? *p1 : p0;
+  q.total0 = p0.tiles_m * p0.tiles_n;
+  q.total = q.total0 + (p1 ? p1->tiles_m * p1->tiles_n : 0);
+  const int grid = ((q.total + 7) / 8) * 8;
+  if (p0.resid)
+    fp8_gemm_kernel<true><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+  else
+    fp8_gemm_kernel<false><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+static int gemm_dispatch(dsx::GemmArgs& p, int64_t M, int64_t N, int64_t K, hipStream_t st) {
+  using namespace dsx;
+  (void)N; (void)K;
+  if (M <= 8) {
+    p.tiles_m = p.tiles_n = 0;
+    return launch_gemv(p, st);
+  }
+  if (p.w_row_scale) return DSX_EBADSHAPE;
+  if (gemm_set_attributes() != DSX_OK) return DSX_ELAUNCH;
+  if (gemm_main_kernel_ok(p)) return launch_main(p, nullptr, st);
+  const int total = p.tiles_m * p.tiles_n;
+  const int grid = ((total + 7) / 8) * 8;
+  fp8_gemm_ragged_k_kernel<<<dim3((unsigned)grid), dim3(256), kStageBytes, st>>>(p);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
@@ -584,4 +654,51 @@ extern "C" int dsx_fp8_gemv_rowscale(const void* a, int64_t lda, const void* w, 
   if (!w_row_scale) return DSX_ENULL;
   p.w_row_scale = w_row_scale;
   return gemm_dispatch(p, M, N, K, (hipStream_t)stream);
+}
+
+static int problem_fill(dsx::GemmArgs& p, const dsx_gemm_problem& d) {
+  int rc = gemm_fill(p, d.a, d.lda, d.w, d.ldw, d.a_scale, d.w_scale, d.bias, d.out, d.ldo, d.M, d.N, d.K);
+  if (rc != DSX_OK) return rc;
+  if (d.resid) {
+    if (d.ldr < d.N || d.rows_per_batch <= 0 || d.rows_per_batch > (1 << 30)) return DSX_EBADSHAPE;
+    if (((uintptr_t)d.resid & 1) || ((uintptr_t)d.gate & 1)) return DSX_EALIGN;
+    p.resid = (const uint16_t*)d.resid;
+    p.gate = (const uint16_t*)d.gate;
+    p.ldr = d.ldr;
+    p.gate_sb = d.gate_sb;
+    p.rows_per_batch = (int)d.rows_per_batch;
+  } else if (d.gate) {
+    return DSX_ENULL;  // a gate without a residual is not an operation of the path
+  }
+  return DSX_OK;
+}
+
+extern "C" int dsx_fp8_gemm_grouped(const dsx_gemm_problem* problems, int count, void* stream) {
+  if (count < 0 || count > DSX_GEMM_GROUP_MAX) return DSX_EBADSHAPE;
+  if (count == 0) return DSX_OK;
+  if (!problems) return DSX_ENULL;
+  dsx::GemmArgs args[DSX_GEMM_GROUP_MAX];
+  for (int i = 0; i < count; ++i) {  // validate everything before anything is launched
+    const int rc = problem_fill(args[i], problems[i]);
+    if (rc != DSX_OK) return rc;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (gemm_set_attributes() != DSX_OK) return DSX_ELAUNCH;
+  bool main_ok[DSX_GEMM_GROUP_MAX];
+  for (int i = 0; i < count; ++i) main_ok[i] = args[i].M > 0 && gemm_main_kernel_ok(args[i]);
+  int i = 0;
+  while (i < count) {
+    if (args[i].M == 0) { ++i; continue; }
+    // pair neighbours that both run on the main kernel and agree on having a residual
+    if (i + 1 < count && main_ok[i] && main_ok[i + 1] && (args[i].resid != nullptr) == (args[i + 1].resid != nullptr)) {
+      const int rc = launch_main(args[i], &args[i + 1], st);
+      if (rc != DSX_OK) return rc;
+      i += 2;
+      continue;
+    }
+    const int rc = gemm_dispatch(args[i], args[i].M, args[i].N, args[i].K, st);
+    if (rc != DSX_OK) return rc;
+    ++i;
+  }
+  return DSX_OK;
 }

@@ -45,9 +45,13 @@ class _Linear:
         self.b = None if bias is None else bias.to(torch.bfloat16).contiguous()
         self.n, self.k = self.w.shape
 
+    def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
+        """Keyword arguments of ``ops.fp8_gemm`` for this layer applied to ``a_q``."""
+        return dict(a_q=a_q, w_q=self.w, a_scale=a_s if self.s is not None else None, w_scale=self.s, bias=self.b,
+                    out=out, resid=resid, gate=gate, rows_per_batch=rows_per_batch)
+
     def __call__(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
-        return ops.fp8_gemm(a_q, self.w, a_s if self.s is not None else None, self.s, self.b, out=out,
-                            resid=resid, gate=gate, rows_per_batch=rows_per_batch)
+        return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch))
 
 
 class FluxDiTRunner:
@@ -151,8 +155,10 @@ class FluxDiTRunner:
         L = self.lin
         qa, sa = self._modulate_q(img, ma[1], ma[0])
         qb, sb = self._modulate_q(txt, mb[1], mb[0])
-        qkv_a = L[pre + "attn.a_to_qkv"](qa.view(-1, d), sa).view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
-        qkv_b = L[pre + "attn.b_to_qkv"](qb.view(-1, d), sb).view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
+        qkv_a, qkv_b = ops.fp8_gemm_grouped([L[pre + "attn.a_to_qkv"].problem(qa.view(-1, d), sa),
+                                             L[pre + "attn.b_to_qkv"].problem(qb.view(-1, d), sb)])
+        qkv_a = qkv_a.view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
+        qkv_b = qkv_b.view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         nw = self.norm_w
@@ -172,22 +178,25 @@ class FluxDiTRunner:
             ops.rmsnorm_rope(ka_, nw[pre + "attn.norm_k_a"], rope, St, EPS, out=ka_)
             ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2),
                                out2=o_a.transpose(1, 2))
-        img = self._stream_tail(pre, "a", img, o_a.view(B * Si, d), ma)
-        txt = self._stream_tail(pre, "b", txt, o_b.view(B * St, d), mb)
-        return img, txt
-
-    def _stream_tail(self, pre, s, x, attn_out, m):
-        """out-projection + gated residual, LN-modulate, MLP + gated residual of one stream (flux_dit.py:226-234)."""
-        L = self.lin
-        B, S, d = x.shape
-        x2 = x.reshape(B * S, d)
-        q, sc = ops.quantize_fp8(attn_out, scaled=self.scaled)
-        x2 = L[pre + f"attn.{s}_to_out"](q, sc, resid=x2, gate=m[2], rows_per_batch=S)
-        q, sc = self._modulate_q(x2.view(B, S, d), m[4], m[3])
-        h = L[pre + f"ff_{s}.0"](q.view(-1, d), sc)
-        q, sc = self._gelu_q(h)
-        x2 = L[pre + f"ff_{s}.2"](q, sc, resid=x2, gate=m[5], rows_per_batch=S)
-        return x2.view(B, S, d)
+        # The two streams run the same sequence on different weights (flux_dit.py:226-234): out-projection +
+        # gated residual, LN-modulate, MLP + gated residual.  Each pair of linears goes out as one grouped
+        # submission so that the 512-token text problem runs beside the image problem instead of after it.
+        xa, xb = img.reshape(B * Si, d), txt.reshape(B * St, d)
+        qa, sa = ops.quantize_fp8(o_a.view(B * Si, d), scaled=self.scaled)
+        qb, sb = ops.quantize_fp8(o_b.view(B * St, d), scaled=self.scaled)
+        xa, xb = ops.fp8_gemm_grouped([
+            L[pre + "attn.a_to_out"].problem(qa, sa, resid=xa, gate=ma[2], rows_per_batch=Si),
+            L[pre + "attn.b_to_out"].problem(qb, sb, resid=xb, gate=mb[2], rows_per_batch=St)])
+        qa, sa = self._modulate_q(xa.view(B, Si, d), ma[4], ma[3])
+        qb, sb = self._modulate_q(xb.view(B, St, d), mb[4], mb[3])
+        ha, hb = ops.fp8_gemm_grouped([L[pre + "ff_a.0"].problem(qa.view(-1, d), sa),
+                                       L[pre + "ff_b.0"].problem(qb.view(-1, d), sb)])
+        qa, sa = self._gelu_q(ha)
+        qb, sb = self._gelu_q(hb)
+        xa, xb = ops.fp8_gemm_grouped([
+            L[pre + "ff_a.2"].problem(qa, sa, resid=xa, gate=ma[5], rows_per_batch=Si),
+            L[pre + "ff_b.2"].problem(qb, sb, resid=xb, gate=mb[5], rows_per_batch=St)])
+        return xa.view(B, Si, d), xb.view(B, St, d)
 
     def _single_block(self, i: int, x, mod, rope):
         """x (B,S,d); mod (B,3d) = shift, scale, gate (transformer_helper.py:34)."""

@@ -86,14 +86,9 @@ def quantize_weight_fp8(w: torch.Tensor, scaled: bool = True):
     return q, scale
 
 
-def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor] = None,
-             w_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
-             out: Optional[torch.Tensor] = None, resid: Optional[torch.Tensor] = None,
-             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None) -> torch.Tensor:
-    """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3.
-
-    With ``resid`` (M,N) the gated residual is fused: out = resid + gate * that, gate (B,N) or None,
-    rows_per_batch = rows of a per batch entry (default: all M rows share gate row 0)."""
+def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, resid=None, gate=None,
+                  rows_per_batch=None):
+    """Validate one GEMM and describe it as a ``dsx_gemm_problem``; returns (problem, out, keep-alive refs)."""
     _require_cuda(a_q, w_q)
     if a_q.dtype != FP8 or w_q.dtype != FP8:
         raise ValueError("fp8_gemm expects float8_e4m3fn operands")
@@ -115,24 +110,57 @@ def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tenso
         bias = bias.contiguous()
     if a_scale is not None:
         a_scale = a_scale.contiguous()
+    gate_sb = 0
+    if resid is not None:
+        if resid.dtype != _BF16 or resid.shape != (M, N) or resid.stride(1) != 1:
+            raise ValueError("fp8_gemm: `resid` must be bf16 (M,N) with unit column stride")
+        if gate is not None:
+            gate = gate.reshape(-1, N)
+            if gate.dtype != _BF16 or gate.stride(1) != 1:
+                gate = gate.to(_BF16).contiguous()
+            gate_sb = gate.stride(0) if gate.shape[0] > 1 else 0
+    elif gate is not None:
+        raise ValueError("fp8_gemm: `gate` needs `resid`")
+    prob = _lib.GemmProblem(
+        a=_ptr(a_q), lda=a_q.stride(0), w=_ptr(w_q), ldw=w_q.stride(0), a_scale=_ptr(a_scale), w_scale=_ptr(w_scale),
+        bias=_ptr(bias), resid=_ptr(resid), ldr=resid.stride(0) if resid is not None else 0, gate=_ptr(gate),
+        gate_sb=gate_sb, rows_per_batch=(rows_per_batch or max(M, 1)), out=_ptr(out), ldo=out.stride(0), M=M, N=N, K=K)
+    return prob, out, (a_q, w_q, a_scale, w_scale, bias, resid, gate)
+
+
+def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor] = None,
+             w_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None, resid: Optional[torch.Tensor] = None,
+             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None) -> torch.Tensor:
+    """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3.
+
+    With ``resid`` (M,N) the gated residual is fused: out = resid + gate * that, gate (B,N) or None,
+    rows_per_batch = rows of a per batch entry (default: all M rows share gate row 0)."""
+    pr, out, _keep = _gemm_problem(a_q, w_q, a_scale, w_scale, bias, out, resid, gate, rows_per_batch)
+    lib = _lib.load()
     if resid is None:
-        rc = _lib.load().dsx_fp8_gemm(_ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale),
-                                      _ptr(w_scale), _ptr(bias), _ptr(out), out.stride(0), M, N, K, _stream())
+        rc = lib.dsx_fp8_gemm(pr.a, pr.lda, pr.w, pr.ldw, pr.a_scale, pr.w_scale, pr.bias, pr.out, pr.ldo,
+                              pr.M, pr.N, pr.K, _stream())
         _lib.check(rc, "dsx_fp8_gemm")
         return out
-    if resid.dtype != _BF16 or resid.shape != (M, N) or resid.stride(1) != 1:
-        raise ValueError("fp8_gemm: `resid` must be bf16 (M,N) with unit column stride")
-    gate_sb = 0
-    if gate is not None:
-        gate = gate.reshape(-1, N)
-        if gate.dtype != _BF16 or gate.stride(1) != 1:
-            gate = gate.to(_BF16).contiguous()
-        gate_sb = gate.stride(0) if gate.shape[0] > 1 else 0
-    rc = _lib.load().dsx_fp8_gemm_gated_residual(
-        _ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale), _ptr(w_scale), _ptr(bias), _ptr(resid),
-        resid.stride(0), _ptr(gate), gate_sb, rows_per_batch or M, _ptr(out), out.stride(0), M, N, K, _stream())
+    rc = lib.dsx_fp8_gemm_gated_residual(pr.a, pr.lda, pr.w, pr.ldw, pr.a_scale, pr.w_scale, pr.bias, pr.resid, pr.ldr,
+                                         pr.gate, pr.gate_sb, pr.rows_per_batch, pr.out, pr.ldo, pr.M, pr.N, pr.K,
+                                         _stream())
     _lib.check(rc, "dsx_fp8_gemm_gated_residual")
     return out
+
+
+def fp8_gemm_grouped(problems):
+    """Several independent GEMMs in one submission; ``problems`` is a list of dicts with the keyword
+    arguments of :func:`fp8_gemm`.  Neighbouring problems share a launch when the kernel allows it
+    (see ``dsx_fp8_gemm_grouped``).  Returns the list of outputs."""
+    if not 0 < len(problems) <= _lib.GEMM_GROUP_MAX:
+        raise ValueError("fp8_gemm_grouped takes 1..%d problems" % _lib.GEMM_GROUP_MAX)
+    built = [_gemm_problem(**kw) for kw in problems]
+    arr = (_lib.GemmProblem * len(built))(*[b[0] for b in built])
+    rc = _lib.load().dsx_fp8_gemm_grouped(arr, len(built), _stream())
+    _lib.check(rc, "dsx_fp8_gemm_grouped")
+    return [b[1] for b in built]
 
 
 def fp8_gemv_rowscale(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor],

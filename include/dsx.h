@@ -102,6 +102,30 @@ int dsx_fp8_gemm_gated_residual(const void* a, int64_t lda, const void* w, int64
                                 int64_t K, void* stream);
 
 /*
+ * Up to DSX_GEMM_GROUP_MAX independent FP8 GEMMs submitted together.  Each problem is exactly
+ * dsx_fp8_gemm (resid == NULL) or dsx_fp8_gemm_gated_residual (resid != NULL) with the same argument
+ * meaning and the same checks; neighbouring problems that both qualify for the 256x256-tile kernel
+ * and agree on having a residual share ONE launch, so a small problem runs on compute units a
+ * large one leaves idle.  The reference issues the image-stream and text-stream linears of a joint
+ * block as separate F.linear calls (diffsynth_engine/models/flux/flux_dit.py:165-171,190-194,
+ * 227-235); this is those pairs.  All problems are validated before anything is launched.
+ */
+#define DSX_GEMM_GROUP_MAX 4
+typedef struct dsx_gemm_problem {
+  const void* a; int64_t lda;          /* (M,K) e4m3 */
+  const void* w; int64_t ldw;          /* (N,K) e4m3 */
+  const float* a_scale;                /* M fp32 or NULL */
+  const float* w_scale;                /* device fp32 scalar or NULL */
+  const void* bias;                    /* N bf16 or NULL */
+  const void* resid; int64_t ldr;      /* (M,N) bf16 or NULL */
+  const void* gate; int64_t gate_sb;   /* (batch,N) bf16 or NULL; needs resid */
+  int64_t rows_per_batch;              /* >= 1 when resid is given */
+  void* out; int64_t ldo;              /* (M,N) bf16 */
+  int64_t M, N, K;
+} dsx_gemm_problem;
+int dsx_fp8_gemm_grouped(const dsx_gemm_problem* problems, int count, void* stream);
+
+/*
  * Small-M (M <= 8) form of dsx_fp8_gemm with one weight scale PER OUTPUT ROW (w_row_scale[n]), so that
  * several Linear layers that consume the same activation can be stacked into one (N_total, K) weight
  * and evaluated by one HBM-bound pass.  Used for the AdaLN projections, which all consume

@@ -181,3 +181,56 @@ def test_fp8_gemv_rowscale_stacks_linears(dev):
                                 torch.cat(bs).to(dev)).cpu()
     want = torch.cat(want, dim=1)
     assert (got.float() - want.float()).abs().max().item() <= 1e-2 * want.float().abs().max().item()
+
+
+def _rand_problem(dev, g, M, N, K, resid=False, bias=True):
+    w = torch.randn(N, K, generator=g) * 0.02
+    x = torch.randn(M, K, generator=g).bfloat16()
+    wq, ws = ofp8.quantize_weight(w)
+    xq, xs = ofp8.quantize_rowwise(x)
+    kw = dict(a_q=xq.to(dev), w_q=wq.to(dev), a_scale=xs.to(dev), w_scale=ws.to(dev),
+              bias=torch.randn(N, generator=g).bfloat16().to(dev) if bias else None)
+    if resid:
+        kw.update(resid=torch.randn(M, N, generator=g).bfloat16().to(dev),
+                  gate=torch.randn(1, N, generator=g).bfloat16().to(dev), rows_per_batch=M)
+    return kw
+
+
+@pytest.mark.parametrize("shapes,resid", [
+    ([(1024, 768, 256), (512, 768, 256)], False),        # image + text stream, same weights' shape
+    ([(1024, 512, 384), (130, 1024, 128)], True),        # different N and K, ragged M, fused residual
+    ([(300, 520, 256), (4, 256, 128), (700, 264, 144), (257, 256, 128)], False),   # gemv + generic-kernel members
+    ([(512, 256, 128)], True),
+])
+def test_fp8_gemm_grouped_equals_separate_launches(dev, shapes, resid):
+    """Problems submitted together give bit-identical results to one dsx_fp8_gemm(_gated_residual) call each,
+    whether neighbours share a launch, fall to the small-M or generic kernel, or stand alone."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(len(shapes) * 17 + shapes[0][0])
+    probs = [_rand_problem(dev, g, M, N, K, resid=resid and M > 8) for (M, N, K) in shapes]
+    want = [ops.fp8_gemm(**p).cpu() for p in probs]
+    got = ops.fp8_gemm_grouped(probs)
+    assert len(got) == len(want)
+    for a, b in zip(got, want):
+        assert torch.equal(a.cpu(), b)
+    # mixed residual / no residual neighbours must not be paired, and still be right
+    if len(shapes) >= 2:
+        mixed = [_rand_problem(dev, g, 512, 256, 128, resid=True), _rand_problem(dev, g, 256, 512, 128, resid=False)]
+        for a, p in zip(ops.fp8_gemm_grouped(mixed), mixed):
+            assert torch.equal(a.cpu(), ops.fp8_gemm(**p).cpu())
+
+
+def test_fp8_gemm_grouped_rejects_bad_arguments(dev):
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    ok = _rand_problem(dev, g, 64, 64, 64)
+    with pytest.raises(ValueError):
+        ops.fp8_gemm_grouped([])
+    with pytest.raises(ValueError):
+        ops.fp8_gemm_grouped([ok] * 5)
+    bad = dict(ok)
+    bad["gate"] = torch.ones(1, 64, dtype=torch.bfloat16, device=dev)   # gate without residual
+    with pytest.raises(ValueError):
+        ops.fp8_gemm_grouped([ok, bad])
