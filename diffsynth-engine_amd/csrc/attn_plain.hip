@@ -5,10 +5,10 @@
 // softmax statistics are lane-local apart from one exchange between the two half-waves).
 //
 // Work split: one workgroup = 8 waves = 256 consecutive queries of one (batch, head); every wave
-// owns 32 queries and needs ~150 VGPRs, so two waves share a SIMD: while one wave's VALU works
-// through exp2/convert/row-sum, the other wave's MFMAs keep the matrix pipe busy.  That costs one
-// LDS operand read per MFMA (128 B/clk per CU at full MFMA rate), which the 256 B/clk LDS of CDNA4
-// carries at half load.
+// owns 32 queries and needs ~230 VGPRs, so two waves share a SIMD and one workgroup fills a CU.
+// While one wave of a SIMD works through exp2/convert/row-sum on the VALU, the other's MFMAs can
+// keep the matrix pipe busy.  That costs one LDS operand read per MFMA, which the 256 B/clk LDS of
+// CDNA4 carries at a quarter load.
 //
 //  * K and V blocks (64 keys) go HBM/L2 -> LDS with global_load_lds_dwordx4, three stages deep,
 //    both stored row-major [key][128 d].  No staging registers, no transposing stores.
@@ -35,19 +35,14 @@ constexpr int QB = 256;  // queries per workgroup (8 waves x 32)
 constexpr int KB = 64;   // keys per block
 constexpr int HD = 128;
 constexpr int kTile = KB * HD * 2;      // 16 KiB
-constexpr int kStage = 2 * kTile;       // K + V
 constexpr int kStages = 3;
+constexpr int kLdsBytes = 2 * kStages * kTile;  // K stages, then V stages
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleThreshold = 64.0f;  // log2 units
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 typedef short v4i16 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ int k_off(int key, int chunk) { return key * 256 + ((chunk ^ (key & 15)) << 4); }
-__device__ __forceinline__ int v_off(int key, int chunk) {
-  return key * 256 + ((chunk ^ ((key & 3) << 2)) << 4);
-}
 
 __device__ __forceinline__ float pair_max(float v) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -82,10 +77,16 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
 
   // ---- async K/V block loads.  One wave instruction = 1 KiB = 4 keys x 256 B; lane l lands at key
   //      l/16, physical chunk l%16.  Per block a wave issues 2 K and 2 V instructions (8 keys).
+  //      Each lane keeps the global address of its 16 bytes of the block last issued; inside a
+  //      segment the next block is one uniform stride further on, so the address arithmetic
+  //      (clamp, segment select, 64-bit multiply) runs only for blocks that touch a segment
+  //      boundary or the ragged end.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_r = lane >> 4, ld_p = lane & 15;
-  auto issue_block = [&](int kb, int stage) {
-    uint8_t* sK = smem + stage * kStage + wave * 2 * 1024;
-    uint8_t* sV = sK + kTile;
+  const uint8_t* kp[2];
+  const uint8_t* vp[2];
+  int ptr_seg = -1;  // segment the pointers advance in; -1: recompute
+  auto set_ptrs = [&](int kb) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int row = (wave * 2 + i) * 4 + ld_r;
@@ -93,18 +94,41 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       if (key >= Skv) key = Skv - 1;
       const int seg = key >= p.skv[0] ? 1 : 0;
       const int64_t lrow = key - (seg ? p.skv[0] : 0);
-      const int ck = ld_p ^ (row & 15);
-      const int cv = ld_p ^ ((row & 3) << 2);
-      __builtin_amdgcn_global_load_lds((gptr_t)(kbase[seg] + lrow * p.k_ss[seg] * 2 + ck * 16),
-                                       (lptr_t)(sK + i * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(vbase[seg] + lrow * p.v_ss[seg] * 2 + cv * 16),
-                                       (lptr_t)(sV + i * 1024), 16, 0, 0);
+      kp[i] = kbase[seg] + lrow * p.k_ss[seg] * 2 + ((ld_p ^ (row & 15)) << 4);
+      vp[i] = vbase[seg] + lrow * p.v_ss[seg] * 2 + ((ld_p ^ ((row & 3) << 2)) << 4);
+    }
+  };
+  auto advance_to = [&](int kb) {  // called with consecutive kb
+    const int64_t k0 = (int64_t)kb * KB;
+    const int lo = k0 >= p.skv[0] ? 1 : 0, hi = k0 + KB - 1 >= p.skv[0] ? 1 : 0;
+    const bool simple = lo == hi && k0 + KB <= Skv;
+    if (simple && ptr_seg == lo) {
+      const int64_t ks = p.k_ss[lo] * (2 * KB), vs = p.v_ss[lo] * (2 * KB);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        kp[i] += ks;
+        vp[i] += vs;
+      }
+    } else {
+      set_ptrs(kb);
+    }
+    ptr_seg = simple ? lo : -1;
+  };
+  auto issue_block = [&](int stage) {
+    uint8_t* sK = smem + stage * kTile + wave_u * 2048;
+    uint8_t* sV = sK + kStages * kTile;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      __builtin_amdgcn_global_load_lds((gptr_t)kp[i], (lptr_t)(sK + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)vp[i], (lptr_t)(sV + i * 1024), 16, 0, 0);
     }
   };
 
   const int nkb = (int)((Skv + KB - 1) / KB);
-  issue_block(0, 0);
-  issue_block(min(1, nkb - 1), 1);
+  advance_to(0);
+  issue_block(0);
+  if (nkb > 1) advance_to(1);
+  issue_block(1);
 
   // ---- Q fragments (B operand of S^T = K Q^T), pre-multiplied by scale*log2(e)
   const float c = p.softmax_scale * kLog2e;
@@ -143,26 +167,42 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  for (int kb = 0; kb < nkb; ++kb) {
-    const int stage = kb % kStages;
+  // LDS read addresses = one lane-dependent VGPR per swizzle class + an immediate: the XOR
+  // swizzles only permute the 16-byte chunk (K) / 64-byte group (V) index by lane-constant bits.
+  //   K fragment (kt, kc): key kt*32 + li, chunk (2kc+g) ^ (li & 15)
+  //   V^T datum (key0 + 32kt + 16ch + 8hi, dt): 64-byte group dt ^ (tr_key & 3), byte tr_dbyte within
+  uint32_t lane_k[8], lane_v[4];
+#pragma unroll
+  for (int kc = 0; kc < 8; ++kc) lane_k[kc] = li * 256 + (((2 * kc + g) ^ (li & 15)) << 4);
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+    lane_v[dt] = kStages * kTile + tr_key * 256 + ((dt ^ (tr_key & 3)) << 6) + tr_dbyte;
+
+  // A 64-key block is three phases: S^T = K Q^T (MFMA), the softmax update (VALU), O^T += V^T P^T
+  // (MFMA), behind one workgroup barrier.  (Running the two waves of a SIMD half a block apart, so
+  // that one wave's VALU phase lies under the other's MFMA phase, was measured 5 % slower.)
+  f32x16 s[2];
+  auto interval_head = [&](int kb) {
     // block kb has landed once at most the 4 loads of block kb+1 are still in flight; the barrier
     // also tells that every wave is done with block kb-1, whose stage block kb+2 will overwrite
     __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
     __builtin_amdgcn_s_barrier();
-    issue_block(min(kb + 2, nkb - 1), (kb + 2) % kStages);
-    const uint8_t* sK = smem + stage * kStage;
-    const uint8_t* sV = sK + kTile;
-
-    // ---- S^T = K (cQ)^T for the 64 keys of the block: two 32-key tiles
-    f32x16 s[2];
+    if (kb + 2 < nkb) advance_to(kb + 2);  // else: re-fetch the last block, nobody reads it
+    issue_block((kb + 2) % kStages);
+  };
+  auto phase_qk = [&](int kb) {
+    const uint8_t* sK = smem + (kb % kStages) * kTile;
 #pragma unroll
     for (int kc = 0; kc < 8; ++kc) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + k_off(kt * 32 + li, 2 * kc + g));
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + lane_k[kc] + kt * 8192);
         s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kc], kc == 0 ? zero16 : s[kt], 0, 0, 0);
       }
     }
+  };
+  uint32_t pw[2][8];  // P as packed bf16, [kt][word]: entries 2w, 2w+1
+  auto phase_softmax = [&](int kb) {
     if ((int64_t)(kb + 1) * KB > Skv) {  // ragged tail of the key axis
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -203,10 +243,8 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
     }
-
     // ---- P = exp2(S'), packed to bf16; the row sum is taken over the ROUNDED values (v_dot2 with
     //      ones), i.e. over exactly the numbers the PV product uses
-    uint32_t pw[2][8];  // [kt][word]: entries 2w, 2w+1
     float lsum = 0.f;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
@@ -218,28 +256,33 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
         lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pw[kt][w]), ones2, lsum, false);
       }
     l_run += lsum;
-
-    // ---- O^T += V^T P^T.  16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
+  };
+  // ---- O^T += V^T P^T.  16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
+  auto phase_pv = [&](int kb) {
+    const uint8_t* sV = smem + (kb % kStages) * kTile;  // lane_v carries the offset of the V region
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int ch = 0; ch < 2; ++ch) {
-        const int key0 = kt * 32 + ch * 16 + tr_key;
         const u32x4 w = {pw[kt][4 * ch + 0], pw[kt][4 * ch + 1], pw[kt][4 * ch + 2], pw[kt][4 * ch + 3]};
         const bf16x8 pf = __builtin_bit_cast(bf16x8, w);
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
-          const int dbyte = dt * 64 + tr_dbyte;
-          const int chunk = dbyte >> 4, within = dbyte & 15;
-          const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) v4i16*)(sV + v_off(key0, chunk) + within));
-          const v4i16 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) v4i16*)(sV + v_off(key0 + 8, chunk) + within));
+          const uint8_t* src = sV + lane_v[dt] + (kt * 32 + ch * 16) * 256;
+          const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)src);
+          const v4i16 hi =
+              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(src + 8 * 256));
           typedef short v8i16 __attribute__((ext_vector_type(8)));
           const v8i16 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, oacc[dt], 0, 0, 0);
         }
       }
+  };
+  for (int kb = 0; kb < nkb; ++kb) {
+    interval_head(kb);
+    phase_qk(kb);
+    phase_softmax(kb);
+    phase_pv(kb);
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain trailing async loads
 
@@ -268,13 +311,13 @@ int launch_attn_plain(const dsx_attn_params& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)attn_plain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kStages * kStage) != hipSuccess)
+                            kLdsBytes) != hipSuccess)
       return DSX_ELAUNCH;
     attr_set = true;
   }
   const int64_t Sq = p.sq[0] + p.sq[1];
   dim3 grid((unsigned)((Sq + QB - 1) / QB), (unsigned)p.heads, (unsigned)p.batch), block(512);
-  attn_plain_kernel<<<grid, block, kStages * kStage, st>>>(p);
+  attn_plain_kernel<<<grid, block, kLdsBytes, st>>>(p);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
