@@ -88,6 +88,8 @@ SIGNATURES = {
     "dsx_rmsnorm_rope": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int64,
                                  c_int64, c_void_p, c_int64, c_int64, c_int64, ctypes.c_int32, ctypes.c_int32,
                                  c_int64, c_void_p]),
+    "dsx_rmsnorm_rope_qk": (c_int, [c_void_p, c_int64, c_int64, ctypes.c_int32, ctypes.c_int32, c_void_p, c_void_p,
+                                    c_float, c_void_p, c_int64, c_int64, ctypes.c_int32, c_int64, c_void_p]),
     "dsx_rmsnorm_rows": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int64, c_void_p, c_int64,
                                  c_int64, c_int64, c_void_p]),
     "dsx_adaln_modulate": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,

@@ -383,6 +383,49 @@ __global__ __launch_bounds__(256) void rmsnorm_rope_kernel(
   if (ok) *reinterpret_cast<u32x4*>(out + b * o_sb + h * o_sh + s * o_ss + c * 8) = o;
 }
 
+
+// RMSNorm + RoPE of the q and k heads of a packed qkv projection, in place, one wavefront per
+// token: a token's heads are contiguous (head h at h*128), q heads first, then k heads.  Sixteen
+// lanes own a head (16 bytes each), so one wave instruction covers four heads; the token's RoPE row
+// and the two norm weights are fetched once and reused for every head.
+__global__ __launch_bounds__(256) void rmsnorm_rope_qk_kernel(
+    uint16_t* x, int64_t x_sb, int64_t x_ss, int heads_q, int heads_k,
+    const uint16_t* __restrict__ wq, const uint16_t* __restrict__ wk, float eps,
+    const float* __restrict__ rope, int64_t rope_sb, int64_t rope_pos0, int64_t seq) {
+  const int lane = threadIdx.x & 63;
+  const int c = lane & 15, hq = lane >> 4;
+  const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int b = blockIdx.y;
+  if (s >= seq) return;  // whole wavefront
+  uint16_t* row = x + b * x_sb + s * x_ss + c * 8;
+  const float* cs = rope ? rope + b * rope_sb + (rope_pos0 + s) * HD + c * 8 : nullptr;
+  const int total = heads_q + heads_k;
+  for (int h0 = 0; h0 < total; h0 += 16) {
+    u32x4 raw[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int h = min(h0 + i * 4 + hq, total - 1);
+      raw[i] = *reinterpret_cast<const u32x4*>(row + h * HD);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int h = h0 + i * 4 + hq;
+      const uint16_t* w = h < heads_q ? wq : wk;
+      float rrms = 1.f;
+      if (w) {
+        float ss = sumsq_chunk(raw[i]);
+        ss += __shfl_xor(ss, 1, 64);
+        ss += __shfl_xor(ss, 2, 64);
+        ss += __shfl_xor(ss, 4, 64);
+        ss += __shfl_xor(ss, 8, 64);
+        rrms = rsqrtf(ss * (1.0f / HD) + eps);
+      }
+      const u32x4 o = norm_rope_chunk(raw[i], w != nullptr, rrms, w ? w + c * 8 : nullptr, cs);
+      if (h < total) *reinterpret_cast<u32x4*>(row + h * HD) = o;
+    }
+  }
+}
+
 }  // namespace dsx
 
 static int check_seg(const void* const* ptr, const int64_t* len) {
@@ -457,5 +500,27 @@ extern "C" int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64
   rmsnorm_rope_kernel<<<grid, block, 0, (hipStream_t)stream>>>(
       (const uint16_t*)x, x_sb, x_sh, x_ss, (const uint16_t*)norm_w, eps, rope, rope_sb, rope_pos0,
       (uint16_t*)out, o_sb, o_sh, o_ss, heads, seq);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int dsx_rmsnorm_rope_qk(void* x, int64_t x_sb, int64_t x_ss, int32_t heads_q, int32_t heads_k,
+                                   const void* q_norm_w, const void* k_norm_w, float eps, const float* rope,
+                                   int64_t rope_sb, int64_t rope_pos0, int32_t batch, int64_t seq,
+                                   void* stream) {
+  using namespace dsx;
+  if (!x) return DSX_ENULL;
+  if (batch <= 0 || heads_q < 0 || heads_k < 0 || heads_q + heads_k <= 0 || heads_q + heads_k > 65535 ||
+      seq < 0 || batch > 65535)
+    return DSX_EBADSHAPE;
+  if (seq > 1 && x_ss < (int64_t)(heads_q + heads_k) * HD) return DSX_EBADSHAPE;
+  if ((x_sb | x_ss) & 7) return DSX_EALIGN;
+  if (((uintptr_t)x & 15) || ((uintptr_t)q_norm_w & 15) || ((uintptr_t)k_norm_w & 15) ||
+      ((uintptr_t)rope & 15) || (rope_sb & 3))
+    return DSX_EALIGN;
+  if (seq == 0) return DSX_OK;
+  dim3 grid((unsigned)((seq + 3) / 4), (unsigned)batch), block(256);
+  rmsnorm_rope_qk_kernel<<<grid, block, 0, (hipStream_t)stream>>>(
+      (uint16_t*)x, x_sb, x_ss, heads_q, heads_k, (const uint16_t*)q_norm_w, (const uint16_t*)k_norm_w, eps,
+      rope, rope_sb, rope_pos0, seq);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }

@@ -457,8 +457,18 @@ __global__ __launch_bounds__(256) void fp8_gemm_ragged_k_kernel(GemmArgs p) {
 // fp32 FMA over the dequantised bytes; the per-row scale form serves several Linear layers
 // stacked into one weight matrix.
 __device__ __forceinline__ void dequant16(const u32x4& v, float* f) {
+  // v_cvt_pk_f32_fp8: two OCP e4m3 bytes of a dword -> two fp32, one VALU instruction per pair
+  // (a bit-twiddling decode costs ~12 per byte and made this kernel VALU-bound)
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-  for (int b = 0; b < 16; ++b) f[b] = e4m3_bits_to_f32((v[b >> 2] >> ((b & 3) * 8)) & 0xffu);
+  for (int w = 0; w < 4; ++w) {
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[w], false);
+    const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)v[w], true);
+    f[4 * w + 0] = lo[0];
+    f[4 * w + 1] = lo[1];
+    f[4 * w + 2] = hi[0];
+    f[4 * w + 3] = hi[1];
+  }
 }
 
 template <int MT>

@@ -157,11 +157,18 @@ class FluxDiTRunner:
         qb, sb = self._modulate_q(txt, mb[1], mb[0])
         qkv_a, qkv_b = ops.fp8_gemm_grouped([L[pre + "attn.a_to_qkv"].problem(qa.view(-1, d), sa),
                                              L[pre + "attn.b_to_qkv"].problem(qb.view(-1, d), sb)])
+        nw = self.norm_w
+        if not self.fuse_rope_in_attention:
+            # RMSNorm + RoPE rewrite q and k in place inside the packed projections (one read + one write of
+            # q and k) so that the attention kernel streams K without re-normalising it once per query tile
+            ops.rmsnorm_rope_qk(qkv_b.view(B, St, 3 * d), HEADS, HEADS, nw[pre + "attn.norm_q_b"],
+                                nw[pre + "attn.norm_k_b"], rope, 0, EPS)
+            ops.rmsnorm_rope_qk(qkv_a.view(B, Si, 3 * d), HEADS, HEADS, nw[pre + "attn.norm_q_a"],
+                                nw[pre + "attn.norm_k_a"], rope, St, EPS)
         qkv_a = qkv_a.view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         qkv_b = qkv_b.view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
-        nw = self.norm_w
         qb_, kb_, vb_ = qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:]
         qa_, ka_, va_ = qkv_a[:, :HEADS], qkv_a[:, HEADS:2 * HEADS], qkv_a[:, 2 * HEADS:]
         if self.fuse_rope_in_attention:
@@ -170,12 +177,6 @@ class FluxDiTRunner:
                                q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
                                out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2))
         else:
-            # RMSNorm + RoPE rewrite q and k in place inside the packed projections (one read + one write of
-            # q and k) so that the attention kernel streams K without re-normalising it once per query tile
-            ops.rmsnorm_rope(qb_, nw[pre + "attn.norm_q_b"], rope, 0, EPS, out=qb_)
-            ops.rmsnorm_rope(kb_, nw[pre + "attn.norm_k_b"], rope, 0, EPS, out=kb_)
-            ops.rmsnorm_rope(qa_, nw[pre + "attn.norm_q_a"], rope, St, EPS, out=qa_)
-            ops.rmsnorm_rope(ka_, nw[pre + "attn.norm_k_a"], rope, St, EPS, out=ka_)
             ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2),
                                out2=o_a.transpose(1, 2))
         # The two streams run the same sequence on different weights (flux_dit.py:226-234): out-projection +
@@ -214,8 +215,8 @@ class FluxDiTRunner:
             ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
                                eps=EPS, out=att.transpose(1, 2))
         else:
-            ops.rmsnorm_rope(q_, nw[pre + "norm_q_a"], rope, 0, EPS, out=q_)
-            ops.rmsnorm_rope(k_, nw[pre + "norm_k_a"], rope, 0, EPS, out=k_)
+            ops.rmsnorm_rope_qk(h.view(B, S, 7 * d), HEADS, HEADS, nw[pre + "norm_q_a"], nw[pre + "norm_k_a"], rope,
+                                0, EPS)
             ops.attention_bhsd(q_, k_, v_, out=att.transpose(1, 2))
         # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
         # parts and emits the e4m3 operand of proj_out with its per-token scale

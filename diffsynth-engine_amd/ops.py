@@ -272,6 +272,29 @@ def rmsnorm_rope(x: torch.Tensor, norm_w: Optional[torch.Tensor], rope: Optional
     return out
 
 
+def rmsnorm_rope_qk(qkv: torch.Tensor, heads_q: int, heads_k: int, q_norm_w: Optional[torch.Tensor],
+                    k_norm_w: Optional[torch.Tensor], rope: Optional[torch.Tensor], pos0: int = 0,
+                    eps: float = 1e-6) -> torch.Tensor:
+    """In-place RMSNorm + RoPE of the q and k heads of a packed projection ``qkv`` (B, S, >= (hq+hk)*128):
+    heads [0,hq) with q_norm_w, [hq,hq+hk) with k_norm_w; the remaining columns (v, ...) are untouched."""
+    _require_cuda(qkv)
+    if qkv.dim() != 3 or qkv.dtype != _BF16 or qkv.stride(2) != 1 or qkv.shape[2] < (heads_q + heads_k) * 128:
+        raise ValueError("rmsnorm_rope_qk expects bf16 (B, S, >= (heads_q+heads_k)*128) with unit column stride")
+    B, S, _ = qkv.shape
+    if q_norm_w is not None:
+        q_norm_w = q_norm_w.to(_BF16).contiguous()
+    if k_norm_w is not None:
+        k_norm_w = k_norm_w.to(_BF16).contiguous()
+    rope_sb = 0
+    if rope is not None:
+        rope = rope.contiguous()
+        rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
+    rc = _lib.load().dsx_rmsnorm_rope_qk(_ptr(qkv), qkv.stride(0), qkv.stride(1), heads_q, heads_k, _ptr(q_norm_w),
+                                         _ptr(k_norm_w), eps, _ptr(rope), rope_sb, pos0, B, S, _stream())
+    _lib.check(rc, "dsx_rmsnorm_rope_qk")
+    return qkv
+
+
 def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, rope: Optional[torch.Tensor] = None,
                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Wan-style RMSNorm over the full last dim of (B,S,D) (or (rows,D)) bf16, optionally followed by RoPE on

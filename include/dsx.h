@@ -187,6 +187,18 @@ int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss, co
                      int64_t seq, void* stream);
 
 /*
+ * The same RMSNorm + RoPE applied in place to the q heads and the k heads of a packed qkv
+ * projection in ONE pass: token row at x + b*x_sb + s*x_ss, head h of that token at + h*128,
+ * heads [0, heads_q) normalised with q_norm_w, heads [heads_q, heads_q + heads_k) with k_norm_w
+ * (either weight may be NULL = no norm), all rotated by the RoPE row rope_pos0 + s (rope NULL = no
+ * rotation).  This is the layout FluxJointAttention.forward / process_attention give q and k
+ * before chunking (flux_dit.py:165-171,297-301: view (B,S,3H,D), norm_q/norm_k, apply_rope).
+ */
+int dsx_rmsnorm_rope_qk(void* x, int64_t x_sb, int64_t x_ss, int32_t heads_q, int32_t heads_k,
+                        const void* q_norm_w, const void* k_norm_w, float eps, const float* rope,
+                        int64_t rope_sb, int64_t rope_pos0, int32_t batch, int64_t seq, void* stream);
+
+/*
  * RMSNorm over whole rows followed by an optional per-head RoPE (head dim 128):
  *   y = bf16( bf16(x * rsqrt(mean(x^2) + eps)) * w ), then pairs (2i,2i+1) of every 128-wide head are rotated by
  *   the (cos, sin) of table row (row % rows_per_batch) [+ rope_sb per batch entry] and rounded to bf16.

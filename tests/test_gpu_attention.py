@@ -149,3 +149,36 @@ def test_bshd_attention_entry_and_errors(dev):
     with pytest.raises(ValueError):
         bad = torch.zeros(1, 1, 8, 64, dtype=torch.bfloat16, device=dev)
         attention(bad, bad, bad)
+
+
+@pytest.mark.parametrize("H,S,extra", [(24, 300, 24 * 128), (3, 17, 0), (5, 64, 128)])
+def test_rmsnorm_rope_qk_in_place_equals_per_tensor_kernel(dev, H, S, extra):
+    """One pass over the packed (B,S,[q heads | k heads | rest]) projection == the single-tensor kernel applied to
+    q and to k separately (same arithmetic), the rest of the row (v, mlp columns) untouched; and the q half
+    agrees with the oracle's RMSNorm -> apply_rope (transformer_helper.py:73-78, flux_dit.py:154-159)."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(H * 100 + S)
+    B, pos0 = 2, 5
+    x = torch.randn(B, S, 2 * H * 128 + extra, generator=g).bfloat16()
+    wq = (1.0 + 0.1 * torch.randn(128, generator=g)).bfloat16()
+    wk = (1.0 + 0.1 * torch.randn(128, generator=g)).bfloat16()
+    ids = torch.zeros(B, pos0 + S, 3)
+    ids[..., 1] = torch.arange(pos0 + S).float() // 7
+    ids[..., 2] = torch.arange(pos0 + S).float() % 7
+    freqs = O.rope_table(ids, (16, 56, 56), 10000)
+    table = ops.rope_table_from_freqs(freqs).to(dev)
+    xd = x.to(dev)
+    heads = xd[:, :, : 2 * H * 128].view(B, S, 2 * H, 128).transpose(1, 2)
+    want_q = ops.rmsnorm_rope(heads[:, :H], wq.to(dev), table, pos0=pos0).cpu()
+    want_k = ops.rmsnorm_rope(heads[:, H:], wk.to(dev), table, pos0=pos0).cpu()
+    got = ops.rmsnorm_rope_qk(xd.clone(), H, H, wq.to(dev), wk.to(dev), table, pos0=pos0).cpu()
+    got_h = got[:, :, : 2 * H * 128].view(B, S, 2 * H, 128).transpose(1, 2)
+    assert torch.equal(got_h[:, :H], want_q)
+    assert torch.equal(got_h[:, H:], want_k)
+    assert torch.equal(got[:, :, 2 * H * 128:], x[:, :, 2 * H * 128:])
+    xq = x[:, :, : H * 128].view(B, S, H, 128).transpose(1, 2)
+    ref = O.apply_rope(O.rms_norm(xq, wq, 1e-6), freqs[:, :, pos0:])
+    diff = (got_h[:, :H].float() - ref.float()).abs()
+    assert (diff > 0).float().mean().item() < 0.01
+    assert diff.max().item() <= 2 ** -6 * ref.float().abs().max().item()
