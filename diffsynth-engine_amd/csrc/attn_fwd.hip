@@ -49,22 +49,20 @@ __device__ __forceinline__ float halfwave_allsum(float v) {
 // RMSNorm + RoPE on 8 consecutive head-dim elements (pairs 4c..4c+3 of the row), given the
 // reciprocal rms of the whole row.  Rounding points follow the bf16 torch sequence:
 // bf16(x * rrms) -> bf16(. * w) -> fp32 rotate -> bf16.
-__device__ __forceinline__ u32x4 norm_rope_chunk(u32x4 raw, bool has_norm, float rrms,
-                                                 const uint16_t* __restrict__ w8,
-                                                 const float* __restrict__ cs8) {
+// Eight consecutive elements of one head: RMSNorm (weights wv, eight bf16) then RoPE (t0, t1 =
+// cos/sin of the four pairs), operands already in registers.
+__device__ __forceinline__ u32x4 norm_rope_regs(u32x4 raw, bool has_norm, float rrms, u32x4 wv, bool has_rope,
+                                                f32x4 t0, f32x4 t1) {
   float v[8];
   v[0] = bf16_lo(raw.x); v[1] = bf16_hi(raw.x); v[2] = bf16_lo(raw.y); v[3] = bf16_hi(raw.y);
   v[4] = bf16_lo(raw.z); v[5] = bf16_hi(raw.z); v[6] = bf16_lo(raw.w); v[7] = bf16_hi(raw.w);
   if (has_norm) {
-    u32x4 wv = *reinterpret_cast<const u32x4*>(w8);
     float wf[8] = {bf16_lo(wv.x), bf16_hi(wv.x), bf16_lo(wv.y), bf16_hi(wv.y),
                    bf16_lo(wv.z), bf16_hi(wv.z), bf16_lo(wv.w), bf16_hi(wv.w)};
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = round_bf16(round_bf16(v[i] * rrms) * wf[i]);
   }
-  if (cs8) {
-    f32x4 t0 = *reinterpret_cast<const f32x4*>(cs8);
-    f32x4 t1 = *reinterpret_cast<const f32x4*>(cs8 + 4);
+  if (has_rope) {
     float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -82,6 +80,18 @@ __device__ __forceinline__ u32x4 norm_rope_chunk(u32x4 raw, bool has_norm, float
   o.z = pack_bf16x2(v[4], v[5]);
   o.w = pack_bf16x2(v[6], v[7]);
   return o;
+}
+
+__device__ __forceinline__ u32x4 norm_rope_chunk(u32x4 raw, bool has_norm, float rrms,
+                                                 const uint16_t* __restrict__ w8,
+                                                 const float* __restrict__ cs8) {
+  const u32x4 wv = has_norm ? *reinterpret_cast<const u32x4*>(w8) : u32x4{0, 0, 0, 0};
+  f32x4 t0 = {0.f, 0.f, 0.f, 0.f}, t1 = t0;
+  if (cs8) {
+    t0 = *reinterpret_cast<const f32x4*>(cs8);
+    t1 = *reinterpret_cast<const f32x4*>(cs8 + 4);
+  }
+  return norm_rope_regs(raw, has_norm, rrms, wv, cs8 != nullptr, t0, t1);
 }
 
 __device__ __forceinline__ float sumsq_chunk(u32x4 raw) {
@@ -400,6 +410,14 @@ __global__ __launch_bounds__(256) void rmsnorm_rope_qk_kernel(
   uint16_t* row = x + b * x_sb + s * x_ss + c * 8;
   const float* cs = rope ? rope + b * rope_sb + (rope_pos0 + s) * HD + c * 8 : nullptr;
   const int total = heads_q + heads_k;
+  const u32x4 zero4 = {0, 0, 0, 0};
+  const u32x4 wvq = wq ? *reinterpret_cast<const u32x4*>(wq + c * 8) : zero4;
+  const u32x4 wvk = wk ? *reinterpret_cast<const u32x4*>(wk + c * 8) : zero4;
+  f32x4 t0 = {0.f, 0.f, 0.f, 0.f}, t1 = t0;
+  if (cs) {
+    t0 = *reinterpret_cast<const f32x4*>(cs);
+    t1 = *reinterpret_cast<const f32x4*>(cs + 4);
+  }
   for (int h0 = 0; h0 < total; h0 += 16) {
     u32x4 raw[4];
 #pragma unroll
@@ -420,7 +438,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rope_qk_kernel(
         ss += __shfl_xor(ss, 8, 64);
         rrms = rsqrtf(ss * (1.0f / HD) + eps);
       }
-      const u32x4 o = norm_rope_chunk(raw[i], w != nullptr, rrms, w ? w + c * 8 : nullptr, cs);
+      const u32x4 o = norm_rope_regs(raw[i], w != nullptr, rrms, h < heads_q ? wvq : wvk, cs != nullptr, t0, t1);
       if (h < total) *reinterpret_cast<u32x4*>(row + h * HD) = o;
     }
   }

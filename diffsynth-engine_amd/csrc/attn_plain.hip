@@ -10,7 +10,7 @@
 // keep the matrix pipe busy.  That costs one LDS operand read per MFMA, which the 256 B/clk LDS of
 // CDNA4 carries at a quarter load.
 //
-//  * K and V blocks (64 keys) go HBM/L2 -> LDS with global_load_lds_dwordx4, three stages deep,
+//  * K and V blocks (64 keys) go HBM/L2 -> LDS with global_load_lds_dwordx4, four stages deep,
 //    both stored row-major [key][128 d].  No staging registers, no transposing stores.
 //  * The V^T operand (8 keys of one d per lane) is read from the row-major V tile with
 //    ds_read_b64_tr_b16: in a 16-lane group, lane i receives element i%4 of the 8-byte datum
@@ -35,7 +35,7 @@ constexpr int QB = 256;  // queries per workgroup (8 waves x 32)
 constexpr int KB = 64;   // keys per block
 constexpr int HD = 128;
 constexpr int kTile = KB * HD * 2;      // 16 KiB
-constexpr int kStages = 3;
+constexpr int kStages = 4;
 constexpr int kLdsBytes = 2 * kStages * kTile;  // K stages, then V stages
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kRescaleThreshold = 64.0f;  // log2 units
@@ -129,6 +129,8 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   issue_block(0);
   if (nkb > 1) advance_to(1);
   issue_block(1);
+  if (nkb > 2) advance_to(2);
+  issue_block(2);
 
   // ---- Q fragments (B operand of S^T = K Q^T), pre-multiplied by scale*log2(e)
   const float c = p.softmax_scale * kLog2e;
@@ -163,8 +165,6 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   const int grp = lane >> 4, j16 = lane & 15;
   const int tr_key = ((grp >> 1) << 2) + (j16 >> 2);    // 4*g of the receiving lanes + key within the quad
   const int tr_dbyte = (grp & 1) * 32 + (j16 & 3) * 8;  // + dt*64, bytes within the 256-byte row
-  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-  const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // LDS read addresses = one lane-dependent VGPR per swizzle class + an immediate: the XOR
@@ -178,37 +178,31 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   for (int dt = 0; dt < 4; ++dt)
     lane_v[dt] = kStages * kTile + tr_key * 256 + ((dt ^ (tr_key & 3)) << 6) + tr_dbyte;
 
-  // A 64-key block is three phases: S^T = K Q^T (MFMA), the softmax update (VALU), O^T += V^T P^T
-  // (MFMA), behind one workgroup barrier.  (Running the two waves of a SIMD half a block apart, so
-  // that one wave's VALU phase lies under the other's MFMA phase, was measured 5 % slower.)
-  f32x16 s[2];
-  auto interval_head = [&](int kb) {
-    // block kb has landed once at most the 4 loads of block kb+1 are still in flight; the barrier
-    // also tells that every wave is done with block kb-1, whose stage block kb+2 will overwrite
-    __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+  // Software pipeline over 64-key blocks.  Interval kb (behind one workgroup barrier) runs
+  //   stage 1:  S(kb+1)^T = K(kb+1) Q^T on the matrix pipe, interleaved instruction by instruction
+  //             with P(kb) = exp2(S(kb)) -> bf16 and its row sums on the VALU (same wave, independent
+  //             registers: the MFMAs execute while the wave issues the exp2 / convert / dot work);
+  //   stage 2:  O^T += V(kb)^T P(kb)^T on the matrix pipe, then the block maximum of S(kb+1) and, when
+  //             it must move, the rescale of the softmax reference (VALU under the tail of the MFMAs).
+  // Without this a wave alternates MFMA-only and VALU-only phases, the two waves of a SIMD do so
+  // in step (they leave the barrier together), and the matrix pipe idles through every softmax.
+  // Four stages of K and V: block kb+1 must have landed when interval kb starts, kb+2 is in flight,
+  // kb+3 is issued into the stage block kb-1 has left.
+  auto interval_head = [&](int kb, int load_stage) {
+    __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4): only block kb+2 may still be in flight
     __builtin_amdgcn_s_barrier();
-    if (kb + 2 < nkb) advance_to(kb + 2);  // else: re-fetch the last block, nobody reads it
-    issue_block((kb + 2) % kStages);
+    if (kb + 3 < nkb) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
+    issue_block(load_stage);
   };
-  auto phase_qk = [&](int kb) {
-    const uint8_t* sK = smem + (kb % kStages) * kTile;
-#pragma unroll
-    for (int kc = 0; kc < 8; ++kc) {
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + lane_k[kc] + kt * 8192);
-        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kc], kc == 0 ? zero16 : s[kt], 0, 0, 0);
-      }
-    }
-  };
-  uint32_t pw[2][8];  // P as packed bf16, [kt][word]: entries 2w, 2w+1
-  auto phase_softmax = [&](int kb) {
-    if ((int64_t)(kb + 1) * KB > Skv) {  // ragged tail of the key axis
+  // softmax reference update for block `blk` whose scores are in s: masks the ragged tail, subtracts
+  // the current reference, and moves it (rescaling O and l) only when the block maximum demands it
+  auto ref_update = [&](f32x16 (&s)[2], int blk) {
+    if ((int64_t)(blk + 1) * KB > Skv) {  // ragged tail of the key axis
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t key = (int64_t)kb * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          const int64_t key = (int64_t)blk * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
           if (key >= Skv) s[kt][r] = -INFINITY;
         }
     }
@@ -218,7 +212,6 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[kt][r] -= m_ref;
     }
-    // ---- block maximum relative to the reference; move the reference only when it must move
     float m0 = max3(s[0][0], s[0][1], s[0][2]);
     float m1 = max3(s[1][0], s[1][1], s[1][2]);
 #pragma unroll
@@ -227,11 +220,11 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       m1 = max3(m1, s[1][r], s[1][r + 1]);
     }
     const float mx = pair_max(max3(m0, m1, fmaxf(s[0][15], s[1][15])));
-    const bool move = mx > kRescaleThreshold || (kb == 0 && mx < -kRescaleThreshold);
+    const bool move = mx > kRescaleThreshold || (blk == 0 && mx < -kRescaleThreshold);
     if (__builtin_amdgcn_ballot_w64(move) != 0) {
       any_ref = true;
-      const float d = kb == 0 ? mx : fmaxf(mx, 0.f);
-      const float alpha = kb == 0 ? 1.0f : __builtin_amdgcn_exp2f(-d);
+      const float d = blk == 0 ? mx : fmaxf(mx, 0.f);
+      const float alpha = blk == 0 ? 1.0f : __builtin_amdgcn_exp2f(-d);
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -243,46 +236,85 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
     }
-    // ---- P = exp2(S'), packed to bf16; the row sum is taken over the ROUNDED values (v_dot2 with
-    //      ones), i.e. over exactly the numbers the PV product uses
-    float lsum = 0.f;
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int w = 0; w < 8; ++w) {
-        const float p0 = __builtin_amdgcn_exp2f(s[kt][2 * w]);
-        const float p1 = __builtin_amdgcn_exp2f(s[kt][2 * w + 1]);
-        pw[kt][w] = pack_bf16x2(p0, p1);
-        lsum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pw[kt][w]), ones2, lsum, false);
-      }
-    l_run += lsum;
   };
-  // ---- O^T += V^T P^T.  16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
-  auto phase_pv = [&](int kb) {
-    const uint8_t* sV = smem + (kb % kStages) * kTile;  // lane_v carries the offset of the V region
+  auto qk = [&](f32x16 (&s)[2], int stage) {
+    const uint8_t* sK = smem + stage * kTile;
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
+    for (int kc = 0; kc < 8; ++kc) {
 #pragma unroll
-      for (int ch = 0; ch < 2; ++ch) {
-        const u32x4 w = {pw[kt][4 * ch + 0], pw[kt][4 * ch + 1], pw[kt][4 * ch + 2], pw[kt][4 * ch + 3]};
-        const bf16x8 pf = __builtin_bit_cast(bf16x8, w);
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          const uint8_t* src = sV + lane_v[dt] + (kt * 32 + ch * 16) * 256;
-          const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)src);
-          const v4i16 hi =
-              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(src + 8 * 256));
-          typedef short v8i16 __attribute__((ext_vector_type(8)));
-          const v8i16 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf, oacc[dt], 0, 0, 0);
-        }
+      for (int kt = 0; kt < 2; ++kt) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + lane_k[kc] + kt * 8192);
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kc], kc == 0 ? zero16 : s[kt], 0, 0, 0);
       }
+    }
   };
-  for (int kb = 0; kb < nkb; ++kb) {
-    interval_head(kb);
-    phase_qk(kb);
-    phase_softmax(kb);
-    phase_pv(kb);
+  // one interval; `stage` (= kb % 4) is a literal so that every LDS offset folds into an immediate
+  auto interval = [&](int kb, int stage, f32x16 (&s_cur)[2], f32x16 (&s_next)[2]) {
+    interval_head(kb, (stage + 3) % kStages);
+    // ---- stage 1: 16 slots, each = [LDS read of the K fragment two MFMAs ahead, one MFMA of
+    //      S(kb+1), two exp2 + one convert + one row-sum step of P(kb)]; sched_barrier pins the order
+    const uint8_t* sK = smem + ((stage + 1) % kStages) * kTile;
+    auto k_frag = [&](int i) {  // MFMA i of the block: k-chunk i/2, key tile i%2
+      return *reinterpret_cast<const bf16x8*>(sK + lane_k[i >> 1] + (i & 1) * 8192);
+    };
+    uint32_t pw[2][8];  // P as packed bf16, [kt][word]: entries 2w, 2w+1
+    float lsum0 = 0.f, lsum1 = 0.f;
+    bf16x8 kf[3];
+    kf[0] = k_frag(0);
+    kf[1] = k_frag(1);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (i + 2 < 16) kf[(i + 2) % 3] = k_frag(i + 2);
+      const int kt = i & 1;
+      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % 3], qf[i >> 1], i < 2 ? zero16 : s_next[kt], 0, 0, 0);
+      // P = exp2(S'), packed to bf16 for the PV product; the row sum adds the fp32 values with plain
+      // v_add_f32 (v_dot2c_f32_bf16 on the packed pair would be one instruction, but it executes on the
+      // matrix pipe and was measured to cost a third of the MFMA rate)
+      const int pk = i >> 3, w = i & 7;
+      const float p0 = __builtin_amdgcn_exp2f(s_cur[pk][2 * w]);
+      const float p1 = __builtin_amdgcn_exp2f(s_cur[pk][2 * w + 1]);
+      pw[pk][w] = pack_bf16x2(p0, p1);
+      lsum0 += p0;
+      lsum1 += p1;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    l_run += lsum0 + lsum1;
+    // ---- stage 2: O^T += V^T P^T, 16 slots = [transposing LDS reads of the V^T operand two MFMAs
+    //      ahead, one MFMA].  16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
+    const uint8_t* sV = smem + stage * kTile;  // lane_v carries the offset of the V region
+    typedef short v8i16 __attribute__((ext_vector_type(8)));
+    auto v_frag = [&](int j) {  // MFMA j: 16-key chunk j/4 (kt = j/8, ch = (j/4)%2), d tile j%4
+      const uint8_t* src = sV + lane_v[j & 3] + (j >> 2) * 16 * 256;
+      const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)src);
+      const v4i16 hi =
+          __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(src + 8 * 256));
+      const v8i16 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      return __builtin_bit_cast(bf16x8, both);
+    };
+    bf16x8 vf[3];
+    vf[0] = v_frag(0);
+    vf[1] = v_frag(1);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (j + 2 < 16) vf[(j + 2) % 3] = v_frag(j + 2);
+      const int kt = j >> 3, ch = (j >> 2) & 1, dt = j & 3;
+      const u32x4 w = {pw[kt][4 * ch + 0], pw[kt][4 * ch + 1], pw[kt][4 * ch + 2], pw[kt][4 * ch + 3]};
+      oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[j % 3], __builtin_bit_cast(bf16x8, w), oacc[dt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kb + 1 < nkb) ref_update(s_next, kb + 1);
+  };
+
+  f32x16 sA[2], sB[2];
+  __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): block 0 has landed
+  __builtin_amdgcn_s_barrier();
+  qk(sA, 0);
+  ref_update(sA, 0);
+  for (int kb = 0; kb < nkb; kb += 4) {
+    interval(kb, 0, sA, sB);
+    if (kb + 1 < nkb) interval(kb + 1, 1, sB, sA);
+    if (kb + 2 < nkb) interval(kb + 2, 2, sA, sB);
+    if (kb + 3 < nkb) interval(kb + 3, 3, sB, sA);
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain trailing async loads
 
