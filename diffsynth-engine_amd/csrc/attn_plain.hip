@@ -60,10 +60,18 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   const int lane = tid & 63;
   const int wave = tid >> 6;  // 0..7
   const int g = lane >> 5, li = lane & 31;
-  const int b = blockIdx.z, h = blockIdx.y;
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of (batch, head,
+  // query block) units so that the query blocks of one head share that head's K/V through ONE L2
+  // (with a plain 3-D grid every XCD ends up fetching every head's K and V).
+  const int nqb = (int)((p.sq[0] + p.sq[1] + QB - 1) / QB);
+  const int total_units = nqb * p.heads * p.batch;
+  const int unit = (int)(blockIdx.x & 7) * ((total_units + 7) >> 3) + (int)(blockIdx.x >> 3);
+  if (unit >= total_units) return;
+  const int qblk = unit % nqb;
+  const int h = (unit / nqb) % p.heads, b = unit / (nqb * p.heads);
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int64_t Skv = p.skv[0] + p.skv[1];
-  const int64_t q0 = (int64_t)blockIdx.x * QB + wave * 32;
+  const int64_t q0 = (int64_t)qblk * QB + wave * 32;
 
   const uint16_t* qbase[2];
   const uint8_t* kbase[2];
@@ -348,7 +356,9 @@ int launch_attn_plain(const dsx_attn_params& p, hipStream_t st) {
     attr_set = true;
   }
   const int64_t Sq = p.sq[0] + p.sq[1];
-  dim3 grid((unsigned)((Sq + QB - 1) / QB), (unsigned)p.heads, (unsigned)p.batch), block(512);
+  const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
+  if (units > (1ll << 30)) return DSX_EBADSHAPE;
+  dim3 grid((unsigned)(((units + 7) / 8) * 8)), block(512);
   attn_plain_kernel<<<grid, block, kLdsBytes, st>>>(p);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
