@@ -104,3 +104,50 @@ def test_zero_gates_make_blocks_identity(dev):
     a = FluxDiTRunner(sd, 2, 2, device=dev)(**inp).cpu()
     b = FluxDiTRunner(sd, 0, 0, device=dev)(**inp).cpu()
     assert torch.equal(a, b)
+
+
+def test_blocks_at_full_sequence_length(dev):
+    """The benchmark's token counts (4096 image + 512 text, 24 heads): one joint block and one single block,
+    teacher-forced, against the oracle evaluated by torch on the device (the CPU would need minutes)."""
+    from diffsynth_engine_amd import ops
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+    from oracle import dit_ops as O
+
+    sd = {k: v.to(dev) for k, v in oflux.init_params(1, 1, dtype=torch.bfloat16, seed=11, bias_std=0.02).items()}
+    P = oflux.Params(sd, "fp8_scaled")
+    R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    g = torch.Generator().manual_seed(12)
+    St, side = 512, 64
+    img = torch.randn(1, side * side, 3072, generator=g).bfloat16().to(dev)
+    txt = torch.randn(1, St, 3072, generator=g).bfloat16().to(dev)
+    cond = torch.randn(1, 3072, generator=g).bfloat16().to(dev)
+    ids = torch.cat([torch.zeros(1, St, 3), oflux.image_ids(2 * side, 2 * side, 1, "cpu", torch.float32)], dim=1)
+    freqs = O.rope_table(ids, oflux.AXES_DIM, oflux.THETA)
+    rope = ops.rope_table_from_freqs(freqs).to(dev)
+    freqs = freqs.to(dev)
+    want_a, want_b = oflux.joint_block(P, 0, img, txt, cond, freqs)
+    mods = R._modulations(cond)
+    got_a, got_b = R._joint_block(0, img, txt, mods["blocks.0.norm1_a.linear"], mods["blocks.0.norm1_b.linear"], rope)
+    assert _cos(got_a, want_a) >= 0.9995 and _cos(got_b, want_b) >= 0.9995, (_cos(got_a, want_a), _cos(got_b, want_b))
+    x = torch.cat([txt, img], dim=1)
+    want = oflux.single_block(P, 0, x, cond, freqs)
+    got = R._single_block(0, x, mods["single_blocks.0.norm.linear"], rope)
+    assert _cos(got, want) >= 0.9995, _cos(got, want)
+    assert torch.isfinite(got.float()).all()
+
+
+def test_batch_of_two_equals_two_single_runs(dev):
+    """A batch of two (the classifier-free-guidance pair, flux_image.py:389-399) gives each entry the result it
+    gets alone: per-entry conditioning, gates and RoPE rows are picked by batch index."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(1, 2, dtype=torch.bfloat16, seed=13, bias_std=0.02)
+    R = FluxDiTRunner(sd, 1, 2, scaled=True, device=dev)
+    a = {k: v.to(dev) for k, v in _inputs(16, 24, seed=14).items()}
+    b = {k: v.to(dev) for k, v in _inputs(16, 24, seed=15).items()}
+    b["timestep"] = torch.tensor([250.0], device=dev)
+    b["guidance"] = torch.tensor([1.0], device=dev)
+    both = {k: torch.cat([a[k], b[k]], dim=0) for k in a}
+    out = R(**both).cpu()
+    assert torch.equal(out[0:1], R(**a).cpu())
+    assert torch.equal(out[1:2], R(**b).cpu())
