@@ -318,6 +318,7 @@ extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale,
                                   int64_t ldq, float* q_scale, int64_t rows, int64_t D,
                                   void* stream) {
   using namespace dsx;
+  if (rows == 0) return DSX_OK;  // an empty batch has no buffers to point at
   if (!x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
   if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || (y && ldy < D) || (q && ldq < D) ||
       rows_per_batch <= 0)
@@ -363,6 +364,7 @@ static int launch_gelu(const void* prefix, int64_t ldp, int64_t Dp, const void* 
 extern "C" int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
                              float* q_scale, int64_t rows, int64_t D, void* stream) {
   using namespace dsx;
+  if (rows == 0) return DSX_OK;  // an empty batch has no buffers to point at
   if (!x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
   if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || (y && ldy < D) || (q && ldq < D))
     return DSX_EBADSHAPE;
@@ -377,6 +379,7 @@ extern "C" int dsx_concat_gelu_tanh(const void* prefix, int64_t ldp, int64_t Dp,
                                     void* y, int64_t ldy, void* q, int64_t ldq, float* q_scale,
                                     int64_t rows, int64_t D, void* stream) {
   using namespace dsx;
+  if (rows == 0) return DSX_OK;
   if (!prefix || !x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
   const int64_t Dt = Dp + D;
   if (rows < 0 || D <= 0 || Dp <= 0 || (D & 7) || (Dp & 7) || Dt > 16384 || ldx < D || ldp < Dp ||
@@ -393,6 +396,7 @@ extern "C" int dsx_gated_residual(const void* x, int64_t ldx, const void* y, int
                                   const void* gate, int64_t gate_sb, int64_t rows_per_batch,
                                   void* out, int64_t ldo, int64_t rows, int64_t D, void* stream) {
   using namespace dsx;
+  if (rows == 0) return DSX_OK;
   if (!x || !y || !out) return DSX_ENULL;
   if (rows < 0 || D <= 0 || (D & 7) || D > (1 << 24) || ldx < D || ldy < D || ldo < D ||
       rows_per_batch <= 0)
@@ -430,6 +434,7 @@ extern "C" int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float
                                 int64_t rope_sb, int64_t rows_per_batch, void* out, int64_t ldo, int64_t rows,
                                 int64_t D, void* stream) {
   using namespace dsx;
+  if (rows == 0) return DSX_OK;
   if (!x || !w || !out) return DSX_ENULL;
   if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || ldo < D || rows_per_batch <= 0 ||
       (rope && (D & 127)))

@@ -598,6 +598,10 @@ static int gemm_dispatch(dsx::GemmArgs& p, int64_t M, int64_t N, int64_t K, hipS
 static int gemm_fill(dsx::GemmArgs& p, const void* a, int64_t lda, const void* w, int64_t ldw,
                      const float* a_scale, const float* w_scale, const void* bias, void* out, int64_t ldo,
                      int64_t M, int64_t N, int64_t K) {
+  if (M == 0 && w) {  // an empty batch: nothing to compute, no activation or output buffer needed
+    p.M = 0;
+    return (N <= 0 || K <= 0) ? DSX_EBADSHAPE : DSX_OK;
+  }
   if (!a || !w || !out) return DSX_ENULL;
   if (M < 0 || N <= 0 || K <= 0 || (K & 15) || lda < K || ldw < K || ldo < N) return DSX_EBADSHAPE;
   if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return DSX_EBADSHAPE;
@@ -640,11 +644,10 @@ extern "C" int dsx_fp8_gemm_gated_residual(const void* a, int64_t lda, const voi
                                            int64_t N, int64_t K, void* stream) {
   dsx::GemmArgs p;
   const int rc = gemm_fill(p, a, lda, w, ldw, a_scale, w_scale, bias, out, ldo, M, N, K);
-  if (rc != DSX_OK) return rc;
+  if (rc != DSX_OK || M == 0) return rc;
   if (!resid) return DSX_ENULL;
   if (ldr < N || rows_per_batch <= 0 || rows_per_batch > (1 << 30)) return DSX_EBADSHAPE;
   if (((uintptr_t)resid & 1) || ((uintptr_t)gate & 1)) return DSX_EALIGN;
-  if (M == 0) return DSX_OK;
   p.resid = (const uint16_t*)resid;
   p.gate = (const uint16_t*)gate;
   p.ldr = ldr;

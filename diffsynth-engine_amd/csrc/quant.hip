@@ -134,6 +134,7 @@ static int launch_quant(const uint16_t* x, int64_t ldx, uint8_t* q, int64_t ldq,
 extern "C" int dsx_quant_fp8_rowwise(const void* x, int64_t ldx, void* q, int64_t ldq,
                                      float* scale_out, int64_t M, int64_t K, void* stream) {
   using namespace dsx;
+  if (M == 0) return DSX_OK;  // an empty batch has no buffers to point at
   if (!x || !q) return DSX_ENULL;
   if (M < 0 || K <= 0 || (K & 7) || K > 512 * 32 || ldx < K || ldq < K) return DSX_EBADSHAPE;
   if ((ldx & 7) || (ldq & 7) || ((uintptr_t)x & 15) || ((uintptr_t)q & 7)) return DSX_EALIGN;

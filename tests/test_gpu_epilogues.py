@@ -162,3 +162,19 @@ def test_adaln_wave_per_row_path_many_rows(dev):
         assert frac < 1e-3 and rel <= 2 ** -6, (D, frac, rel)
         wq, ws = ofp8.quantize_rowwise(y.cpu().reshape(-1, D), scaled=True)
         assert torch.equal(qs.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8).reshape(-1, D), wq.view(torch.uint8))
+
+
+def test_empty_inputs_are_accepted(dev):
+    """Zero rows are a valid (empty) workload for every row kernel and for the GEMM: nothing is launched and
+    an empty output comes back (the reference's torch ops accept empty batches the same way)."""
+    from diffsynth_engine_amd import ops
+
+    x = torch.zeros(0, 3072, dtype=torch.bfloat16, device=dev)
+    q, s = ops.quantize_fp8(x, scaled=True)
+    assert q.shape == (0, 3072) and s.shape == (0,)
+    w = torch.zeros(256, 3072, dtype=torch.bfloat16, device=dev)
+    wq, ws = ops.quantize_weight_fp8(w)
+    assert ops.fp8_gemm(q, wq, s, ws, None).shape == (0, 256)
+    assert ops.gelu_tanh(x).shape == (0, 3072)
+    mod = torch.zeros(1, 3072, dtype=torch.bfloat16, device=dev)
+    assert ops.adaln_modulate(x.view(1, 0, 3072), mod, mod, 1e-6).shape == (1, 0, 3072)
