@@ -28,16 +28,17 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
   return u >> 16;
 }
 
-// Round an fp32 value to the nearest bf16 and return it widened again (an in-register
-// "rounding point" reproducing an intermediate bf16 tensor of the torch op sequence).
-__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
-
 // Two fp32 -> packed bf16 pair with the hardware converter (v_cvt_pk_bf16_f32, RNE).
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
   bf16x2 v = {(__bf16)lo, (__bf16)hi};
   return __builtin_bit_cast(uint32_t, v);
 }
+
+// Round an fp32 value to the nearest bf16 and return it widened again (an in-register
+// "rounding point" reproducing an intermediate bf16 tensor of the torch op sequence): the hardware
+// converter and a shift, two instructions where the integer formulation takes seven.
+__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(pack_bf16x2(f, f) << 16); }
 
 // Unpack the two bf16 halves of a 32-bit word.
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
@@ -94,6 +95,16 @@ __device__ __forceinline__ float wave_sum(float v) {
 // tanh-GELU in fp32 with the expression torch evaluates for approximate="tanh":
 // 0.5 * x * (1 + tanh(sqrt(2/pi) * (x + 0.044715 x^3))).  tanh(u) = 1 - 2/(exp(2u)+1) has an
 // absolute error of about one fp32 ulp of 1.0, like a library tanhf, and saturates to +-1 cleanly.
+// Four fp32 -> four OCP e4m3 bytes of one dword with the hardware converter (v_cvt_pk_fp8_f32, RNE,
+// two values per instruction).  For |v| <= 448 the result equals f32_to_e4m3_bits; beyond that the
+// converter's out-of-range result is the hardware's, so callers that must reproduce torch's bare cast
+// (NaN from 465 on) use this only on values already scaled into range.
+__device__ __forceinline__ uint32_t pack_e4m3x4_inrange(float a, float b, float c, float d) {
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  return (uint32_t)w;
+}
+
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
   const float kBeta = 0.7978845608028654f;  // sqrt(2/pi)
   const float kKappa = 0.044715f;

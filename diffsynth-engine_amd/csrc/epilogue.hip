@@ -43,13 +43,10 @@ __device__ __forceinline__ u32x4 pack8(const float* v) {
   o.w = pack_bf16x2(v[6], v[7]);
   return o;
 }
-__device__ __forceinline__ u32x2 quant8(const float* v, float inv) {
-  uint32_t b[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) b[i] = f32_to_e4m3_bits(v[i] * inv);
+__device__ __forceinline__ u32x2 quant8(const float* v, float inv) {  // |v * inv| <= 448 by construction
   u32x2 r;
-  r.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
-  r.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+  r.x = pack_e4m3x4_inrange(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+  r.y = pack_e4m3x4_inrange(v[4] * inv, v[5] * inv, v[6] * inv, v[7] * inv);
   return r;
 }
 

@@ -5,9 +5,16 @@
 
 namespace dsx {
 
-// Quantise 8 floats (already divided by the scale) to 8 e4m3 bytes.
+// Quantise 8 floats (already divided by the scale) to 8 e4m3 bytes.  IN_RANGE: every |v| <= 448
+// (scaled quantisation), so the hardware converter applies.
+template <bool IN_RANGE>
 __device__ __forceinline__ u32x2 pack_e4m3x8(const float* v) {
   u32x2 r;
+  if (IN_RANGE) {
+    r.x = pack_e4m3x4_inrange(v[0], v[1], v[2], v[3]);
+    r.y = pack_e4m3x4_inrange(v[4], v[5], v[6], v[7]);
+    return r;
+  }
   r.x = f32_to_e4m3_bits(v[0]) | (f32_to_e4m3_bits(v[1]) << 8) | (f32_to_e4m3_bits(v[2]) << 16) |
         (f32_to_e4m3_bits(v[3]) << 24);
   r.y = f32_to_e4m3_bits(v[4]) | (f32_to_e4m3_bits(v[5]) << 8) | (f32_to_e4m3_bits(v[6]) << 16) |
@@ -71,7 +78,7 @@ __global__ __launch_bounds__(256) void quant_rowwise_kernel(const uint16_t* __re
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = v[j] * inv;
       }
-      qr[c] = pack_e4m3x8(v);
+      qr[c] = pack_e4m3x8<SCALED>(v);
     }
   }
 }
