@@ -106,12 +106,13 @@ __device__ __forceinline__ uint32_t pack_e4m3x4_inrange(float a, float b, float 
 }
 
 __device__ __forceinline__ float gelu_tanh_f32(float x) {
-  const float kBeta = 0.7978845608028654f;  // sqrt(2/pi)
-  const float kKappa = 0.044715f;
-  const float u = kBeta * (x + kKappa * (x * x * x));
-  const float e = __builtin_amdgcn_exp2f(u * 2.8853900817779268f);  // exp(2u)
-  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
-  return 0.5f * x * (1.0f + t);
+  // 0.5 x (1 + tanh(u)), u = sqrt(2/pi) (x + 0.044715 x^3), written as x / (1 + exp(-2u)): seven VALU
+  // instructions (two transcendental), no cancellation in the negative tail, no overflow (x * 0 for
+  // x -> -inf).  Agrees with torch's fp32 evaluation of the tanh form to within its own rounding noise.
+  const float c1 = -2.0f * 1.4426950408889634f * 0.7978845608028654f;
+  const float c3 = c1 * 0.044715f;
+  const float a = x * __builtin_fmaf(x * x, c3, c1);  // -2u * log2(e)
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a));
 }
 
 // Exactly rounded a*b + c*d with every operation rounded on its own (no FMA contraction), the
