@@ -151,3 +151,34 @@ def test_batch_of_two_equals_two_single_runs(dev):
     out = R(**both).cpu()
     assert torch.equal(out[0:1], R(**a).cpu())
     assert torch.equal(out[1:2], R(**b).cpu())
+
+
+def test_three_step_denoising_loop(dev):
+    """Scheduler -> [DiT runner -> Euler step] x 3 on the device, as FluxImagePipeline's loop chains them
+    (flux_image.py:505-530: timestep = sigma * 1000 into the DiT, latents <- sampler.step), against the same
+    loop built from the oracle's forward and sampler step."""
+    from diffsynth_engine_amd import sampler as host
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+    from oracle import sampler as osamp
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=21, bias_std=0.02)
+    sd_dev = {k: v.to(dev) for k, v in sd.items()}
+    R = FluxDiTRunner(sd_dev, 1, 1, scaled=True, device=dev)
+    inp = {k: v.to(dev) for k, v in _inputs(16, 24, seed=22).items()}
+    sched = host.RecifitedFlowScheduler(shift=3.0, use_dynamic_shifting=True)
+    sigmas, timesteps = sched.schedule(3, mu=host.calculate_shift(64))
+    want_sig, want_ts = osamp.recified_flow_schedule(3, mu=osamp.calculate_shift(64), use_dynamic_shifting=True)
+    assert torch.equal(sigmas, want_sig) and torch.equal(timesteps, want_ts)
+    smp = host.FlowMatchEulerSampler()
+    smp.initialize(None, timesteps, sigmas, None)
+    P = oflux.Params(sd_dev, "fp8_scaled")
+    lat = inp["hidden_states"]
+    lat_o = lat.clone()
+    for i in range(3):
+        t = timesteps[i : i + 1].to(dev)
+        step_in = dict(inp, hidden_states=lat, timestep=t)
+        lat = smp.step(lat, R(**step_in), i)
+        v_o = oflux.flux_dit_forward(P, **dict(inp, hidden_states=lat_o, timestep=t), num_double=1, num_single=1)
+        lat_o = osamp.flow_match_euler_step(lat_o, v_o, sigmas, i)
+    assert torch.isfinite(lat.float()).all()
+    assert _cos(lat, lat_o) >= 0.999, _cos(lat, lat_o)
