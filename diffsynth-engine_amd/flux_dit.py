@@ -33,9 +33,9 @@ EPS = 1e-6
 
 
 class _Linear:
-    """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias."""
+    """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias, plus optional unfused LoRA pairs."""
 
-    __slots__ = ("w", "s", "b", "n", "k")
+    __slots__ = ("w", "s", "b", "n", "k", "loras", "scaled")
 
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], scaled: bool):
         if weight.dtype == ops.FP8:
@@ -44,6 +44,23 @@ class _Linear:
             self.w, self.s = ops.quantize_weight_fp8(weight, scaled=scaled)
         self.b = None if bias is None else bias.to(torch.bfloat16).contiguous()
         self.n, self.k = self.w.shape
+        self.loras = []  # (down_q (r,K), down_scale, up_q (N,r), up_scale * coefficient)
+        self.scaled = scaled
+
+    def add_lora(self, down: torch.Tensor, up: torch.Tensor, coef: float):
+        """Unfused low-rank update y += coef * up(down(x)) (models/basic/lora.py:29-32,137-141); both factors are
+        stored as e4m3 like every other Linear under fp8 inference.  The rank is zero-padded to a multiple of 16
+        (the GEMM's K granularity) and the coefficient is folded into the up factor's scale."""
+        r = down.shape[0]
+        rp = (r + 15) // 16 * 16
+        dev = self.w.device
+        d = torch.zeros((rp, self.k), dtype=torch.bfloat16, device=dev)
+        d[:r] = down.to(dev, torch.bfloat16)
+        u = torch.zeros((self.n, rp), dtype=torch.bfloat16, device=dev)
+        u[:, :r] = up.to(dev, torch.bfloat16)
+        dq, ds = ops.quantize_weight_fp8(d, scaled=True)
+        uq, us = ops.quantize_weight_fp8(u, scaled=True)
+        self.loras.append((dq, ds, uq, (us * coef).float()))
 
     def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
         """Keyword arguments of ``ops.fp8_gemm`` for this layer applied to ``a_q``."""
@@ -51,7 +68,29 @@ class _Linear:
                     out=out, resid=resid, gate=gate, rows_per_batch=rows_per_batch)
 
     def __call__(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
-        return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch))
+        if not self.loras:
+            return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch))
+        lows = []
+        for dq, ds, uq, us in self.loras:
+            hq, hs = ops.quantize_fp8(ops.fp8_gemm(a_q, dq, a_s, ds, None), scaled=True)
+            lows.append((hq, hs, uq, us))
+        if resid is None:  # y = main + sum(lora): the low-rank products are added by residual epilogues
+            y = ops.fp8_gemm(**self.problem(a_q, a_s, out))
+            for hq, hs, uq, us in lows:
+                ops.fp8_gemm(hq, uq, hs, us, None, resid=y, out=y)
+            return y
+        # resid + gate*(main + lora) = (resid + gate*lora) + gate*main: every term rides a GEMM epilogue
+        acc = resid
+        for hq, hs, uq, us in lows:
+            acc = ops.fp8_gemm(hq, uq, hs, us, None, resid=acc, gate=gate, rows_per_batch=rows_per_batch)
+        return ops.fp8_gemm(**self.problem(a_q, a_s, out, acc, gate, rows_per_batch))
+
+
+def _gemm_pair(la: "_Linear", pa: dict, lb: "_Linear", pb: dict):
+    """Two independent linears (image and text stream): one grouped submission unless a LoRA is attached."""
+    if la.loras or lb.loras:
+        return la(**pa), lb(**pb)
+    return ops.fp8_gemm_grouped([la.problem(**pa), lb.problem(**pb)])
 
 
 class FluxDiTRunner:
@@ -99,6 +138,11 @@ class FluxDiTRunner:
         self.mod_w = torch.cat(ws, dim=0)
         self.mod_row_scale = torch.cat(ss).contiguous()
         self.mod_bias = torch.cat(bs).contiguous()
+
+    def add_lora(self, name: str, down: torch.Tensor, up: torch.Tensor, coef: float = 1.0):
+        """Attach an unfused LoRA (``coef`` = scale * alpha / rank) to the Linear called ``name``; the AdaLN
+        projections are stacked at construction and take no LoRA here."""
+        self.lin[name].add_lora(down, up, coef)
 
     # ------------------------------------------------------------------ small helpers
     def _linear_bf16(self, x: torch.Tensor, name: str) -> torch.Tensor:
@@ -155,8 +199,8 @@ class FluxDiTRunner:
         L = self.lin
         qa, sa = self._modulate_q(img, ma[1], ma[0])
         qb, sb = self._modulate_q(txt, mb[1], mb[0])
-        qkv_a, qkv_b = ops.fp8_gemm_grouped([L[pre + "attn.a_to_qkv"].problem(qa.view(-1, d), sa),
-                                             L[pre + "attn.b_to_qkv"].problem(qb.view(-1, d), sb)])
+        qkv_a, qkv_b = _gemm_pair(L[pre + "attn.a_to_qkv"], dict(a_q=qa.view(-1, d), a_s=sa),
+                                  L[pre + "attn.b_to_qkv"], dict(a_q=qb.view(-1, d), a_s=sb))
         nw = self.norm_w
         if not self.fuse_rope_in_attention:
             # RMSNorm + RoPE rewrite q and k in place inside the packed projections (one read + one write of
@@ -185,18 +229,16 @@ class FluxDiTRunner:
         xa, xb = img.reshape(B * Si, d), txt.reshape(B * St, d)
         qa, sa = ops.quantize_fp8(o_a.view(B * Si, d), scaled=self.scaled)
         qb, sb = ops.quantize_fp8(o_b.view(B * St, d), scaled=self.scaled)
-        xa, xb = ops.fp8_gemm_grouped([
-            L[pre + "attn.a_to_out"].problem(qa, sa, resid=xa, gate=ma[2], rows_per_batch=Si),
-            L[pre + "attn.b_to_out"].problem(qb, sb, resid=xb, gate=mb[2], rows_per_batch=St)])
+        xa, xb = _gemm_pair(L[pre + "attn.a_to_out"], dict(a_q=qa, a_s=sa, resid=xa, gate=ma[2], rows_per_batch=Si),
+                            L[pre + "attn.b_to_out"], dict(a_q=qb, a_s=sb, resid=xb, gate=mb[2], rows_per_batch=St))
         qa, sa = self._modulate_q(xa.view(B, Si, d), ma[4], ma[3])
         qb, sb = self._modulate_q(xb.view(B, St, d), mb[4], mb[3])
-        ha, hb = ops.fp8_gemm_grouped([L[pre + "ff_a.0"].problem(qa.view(-1, d), sa),
-                                       L[pre + "ff_b.0"].problem(qb.view(-1, d), sb)])
+        ha, hb = _gemm_pair(L[pre + "ff_a.0"], dict(a_q=qa.view(-1, d), a_s=sa),
+                            L[pre + "ff_b.0"], dict(a_q=qb.view(-1, d), a_s=sb))
         qa, sa = self._gelu_q(ha)
         qb, sb = self._gelu_q(hb)
-        xa, xb = ops.fp8_gemm_grouped([
-            L[pre + "ff_a.2"].problem(qa, sa, resid=xa, gate=ma[5], rows_per_batch=Si),
-            L[pre + "ff_b.2"].problem(qb, sb, resid=xb, gate=mb[5], rows_per_batch=St)])
+        xa, xb = _gemm_pair(L[pre + "ff_a.2"], dict(a_q=qa, a_s=sa, resid=xa, gate=ma[5], rows_per_batch=Si),
+                            L[pre + "ff_b.2"], dict(a_q=qb, a_s=sb, resid=xb, gate=mb[5], rows_per_batch=St))
         return xa.view(B, Si, d), xb.view(B, St, d)
 
     def _single_block(self, i: int, x, mod, rope):

@@ -32,6 +32,7 @@ class Params:
         self.t = tensors
         self.linear_mode = linear_mode
         self._q = {}
+        self.lora = {}  # layer name -> list of (down (r,K), up (N,r), coefficient)
         # geometry: Flux.1-dev's unless a test builds a reduced model (flux_dit.py:343,352-356)
         self.heads, self.head_dim, self.axes_dim = heads, head_dim, tuple(axes_dim)
 
@@ -39,13 +40,20 @@ class Params:
         return self.t[k]
 
     def linear(self, x, name):
-        w = self.t[name + ".weight"]
-        b = self.t.get(name + ".bias")
+        """nn.Linear, or LoRALinear.forward when low-rank pairs are attached (models/basic/lora.py:29-32,137-141:
+        w_x = linear(x); w_x += scale * alpha / rank * up(down(x)), every F.linear through the fp8 patch)."""
+        y = self._linear(x, self.t[name + ".weight"], self.t.get(name + ".bias"), name)
+        for j, (down, up, coef) in enumerate(self.lora.get(name, ())):
+            h = self._linear(x, down, None, f"{name}#lora{j}.down")
+            y = y + coef * self._linear(h, up, None, f"{name}#lora{j}.up")
+        return y
+
+    def _linear(self, x, w, b, key):
         if self.linear_mode == "plain":
             return F.linear(x, w, b)
-        if name not in self._q:
-            self._q[name] = fp8.quantize_weight(w, scaled=self.linear_mode == "fp8_scaled")
-        w_q, w_s = self._q[name]
+        if key not in self._q:
+            self._q[key] = fp8.quantize_weight(w, scaled=self.linear_mode == "fp8_scaled")
+        w_q, w_s = self._q[key]
         return fp8.fp8_linear(x, w_q, w_s, b)
 
 

@@ -182,3 +182,44 @@ def test_three_step_denoising_loop(dev):
         lat_o = osamp.flow_match_euler_step(lat_o, v_o, sigmas, i)
     assert torch.isfinite(lat.float()).all()
     assert _cos(lat, lat_o) >= 0.999, _cos(lat, lat_o)
+
+
+def test_unfused_lora_on_runner_linears(dev):
+    """LoRALinear.forward (models/basic/lora.py:137-141) on a plain linear (qkv), on linears whose output enters
+    a gated residual (out-projection, single-block proj_out) and on both streams of a joint block: runner with
+    attached low-rank pairs against the oracle with the same pairs."""
+    from diffsynth_engine_amd import ops
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+    from oracle import dit_ops as O
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=31, bias_std=0.02)
+    P = oflux.Params(sd, "fp8_scaled")
+    R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    g = torch.Generator().manual_seed(32)
+    targets = {"blocks.0.attn.a_to_qkv": 16, "blocks.0.attn.b_to_out": 8, "blocks.0.ff_a.2": 32,
+               "single_blocks.0.to_qkv_mlp": 16, "single_blocks.0.proj_out": 4}
+    for name, r in targets.items():
+        n, k = sd[name + ".weight"].shape
+        down = (torch.randn(r, k, generator=g) * 0.05).bfloat16()
+        up = (torch.randn(n, r, generator=g) * 0.05).bfloat16()
+        P.lora[name] = [(down, up, 0.5)]
+        R.add_lora(name, down, up, 0.5)
+    St, side = 40, 12
+    img = torch.randn(1, side * side, 3072, generator=g).bfloat16()
+    txt = torch.randn(1, St, 3072, generator=g).bfloat16()
+    cond = torch.randn(1, 3072, generator=g).bfloat16()
+    ids = torch.cat([torch.zeros(1, St, 3), oflux.image_ids(2 * side, 2 * side, 1, "cpu", torch.float32)], dim=1)
+    freqs = O.rope_table(ids, oflux.AXES_DIM, oflux.THETA)
+    rope = ops.rope_table_from_freqs(freqs).to(dev)
+    want_a, want_b = oflux.joint_block(P, 0, img, txt, cond, freqs)
+    base = oflux.Params(sd, "fp8_scaled")
+    base_a, _ = oflux.joint_block(base, 0, img, txt, cond, freqs)
+    assert _cos(base_a, want_a) < 0.9999  # the low-rank terms matter in this set-up
+    mods = R._modulations(cond.to(dev))
+    got_a, got_b = R._joint_block(0, img.to(dev), txt.to(dev), mods["blocks.0.norm1_a.linear"],
+                                  mods["blocks.0.norm1_b.linear"], rope)
+    assert _cos(got_a, want_a) >= 0.9995 and _cos(got_b, want_b) >= 0.9995, (_cos(got_a, want_a), _cos(got_b, want_b))
+    x = torch.cat([txt, img], dim=1)
+    want = oflux.single_block(P, 0, x, cond, freqs)
+    got = R._single_block(0, x.to(dev), mods["single_blocks.0.norm.linear"], rope)
+    assert _cos(got, want) >= 0.9995, _cos(got, want)
