@@ -20,6 +20,7 @@ DSX_EALIGN = -2
 DSX_EARCH = -3
 DSX_ELAUNCH = -4
 DSX_ENULL = -5
+ABI_VERSION = 2
 
 
 class AttnParams(ctypes.Structure):
@@ -44,6 +45,8 @@ class AttnParams(ctypes.Structure):
         ("k_norm_w", c_void_p * 2),
         ("norm_eps", c_float),
         ("reserved", ctypes.c_int32),
+        ("workspace", c_void_p),
+        ("workspace_bytes", c_int64),
     ]
 
 
@@ -122,8 +125,8 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
-    if lib.dsx_abi_version() != 1:
-        raise ImportError("libdsx.so ABI version %d, expected 1" % lib.dsx_abi_version())
+    if lib.dsx_abi_version() != ABI_VERSION:
+        raise ImportError("libdsx.so ABI version %d, expected %d" % (lib.dsx_abi_version(), ABI_VERSION))
     _lib = lib
     return lib
 

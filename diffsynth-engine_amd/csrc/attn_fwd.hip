@@ -481,6 +481,47 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
 
   if (!fused) return launch_attn_plain(*p, (hipStream_t)stream);
 
+  // With caller scratch: normalise / rotate q and k once into it, then run the plain kernel on the copies.
+  const int64_t ws_need = 2 * (int64_t)p->batch * p->heads * (Sq + Skv) * HD;
+  if (p->workspace && p->workspace_bytes >= ws_need) {
+    if ((uintptr_t)p->workspace & 15) return DSX_EALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    dsx_attn_params t = *p;
+    uint16_t* wq = (uint16_t*)p->workspace;
+    uint16_t* wk = wq + (int64_t)p->batch * p->heads * Sq * HD;
+    for (int which = 0; which < 2; ++which) {  // 0: q, 1: k
+      uint16_t* base = which ? wk : wq;
+      const int64_t rows = which ? Skv : Sq;
+      const int64_t o_sh = rows * HD, o_sb = (int64_t)p->heads * rows * HD;
+      int64_t row0 = 0;
+      for (int g = 0; g < 2; ++g) {
+        const int64_t n = which ? p->skv[g] : p->sq[g];
+        uint16_t* dst = base + row0 * HD;
+        if (n > 0) {
+          const void* src = which ? p->k[g] : p->q[g];
+          const int64_t sb = which ? p->k_sb[g] : p->q_sb[g], sh = which ? p->k_sh[g] : p->q_sh[g],
+                        ss = which ? p->k_ss[g] : p->q_ss[g];
+          dim3 grid((unsigned)((n + 15) / 16), (unsigned)p->heads, (unsigned)p->batch), block(256);
+          rmsnorm_rope_kernel<<<grid, block, 0, st>>>(
+              (const uint16_t*)src, sb, sh, ss, (const uint16_t*)(which ? p->k_norm_w[g] : p->q_norm_w[g]),
+              p->norm_eps, p->rope, p->rope_sb, row0, dst, o_sb, o_sh, HD, p->heads, n);
+        }
+        if (which) {
+          t.k[g] = n > 0 ? dst : nullptr;
+          t.k_sb[g] = o_sb; t.k_sh[g] = o_sh; t.k_ss[g] = HD;
+        } else {
+          t.q[g] = n > 0 ? dst : nullptr;
+          t.q_sb[g] = o_sb; t.q_sh[g] = o_sh; t.q_ss[g] = HD;
+        }
+        row0 += n;
+      }
+    }
+    if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
+    t.rope = nullptr;
+    t.q_norm_w[0] = t.q_norm_w[1] = t.k_norm_w[0] = t.k_norm_w[1] = nullptr;
+    return launch_attn_plain(t, st);
+  }
+
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)attn_fwd_kernel<false>,

@@ -219,7 +219,7 @@ class FluxDiTRunner:
             ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, rope=rope,
                                q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
                                q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
-                               out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2))
+                               out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2), in_kernel=True)
         else:
             ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2),
                                out2=o_a.transpose(1, 2))
@@ -255,7 +255,7 @@ class FluxDiTRunner:
         q_, k_, v_ = qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:]
         if self.fuse_rope_in_attention:
             ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
-                               eps=EPS, out=att.transpose(1, 2))
+                               eps=EPS, out=att.transpose(1, 2), in_kernel=True)
         else:
             ops.rmsnorm_rope_qk(h.view(B, S, 7 * d), HEADS, HEADS, nw[pre + "norm_q_a"], nw[pre + "norm_k_a"], rope,
                                 0, EPS)

@@ -192,13 +192,15 @@ def rope_table_from_freqs(freqs: torch.Tensor) -> torch.Tensor:
 def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float] = None,
                    rope: Optional[torch.Tensor] = None, q_norm_w=None, k_norm_w=None, q2_norm_w=None,
                    k2_norm_w=None, eps: float = 1e-6, out: Optional[torch.Tensor] = None,
-                   out2: Optional[torch.Tensor] = None):
+                   out2: Optional[torch.Tensor] = None, in_kernel: bool = False):
     """softmax(q k^T * scale) v over the concatenation [segment 1, segment 2] of rows.
 
     q, k, v: (B,H,S,128) bf16 views with unit stride in the last dim (any other strides).
     q2/k2/v2: optional second segment (same strides as the first), appended after the first.
     rope: optional (B or 1, Sq, 64, 2) fp32 (cos, sin) table applied in-kernel to q and k;
-    *_norm_w: optional (128,) bf16 RMSNorm weights applied in-kernel before RoPE.
+    *_norm_w: optional (128,) bf16 RMSNorm weights applied before RoPE.
+    in_kernel: apply RoPE / RMSNorm inside the attention kernel as tiles are loaded (every query block then
+    repeats the work on K); default: normalise / rotate q and k once into a scratch buffer allocated here.
     Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).
     """
     _require_cuda(q, k, v)
@@ -245,6 +247,10 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
                 keep.append(w)
                 getattr(P, name)[i] = _ptr(w)
     P.norm_eps = eps
+    if keep and not in_kernel:
+        ws = torch.empty(2 * B * H * (S1 + S2 + Skv1 + Skv2) * D, dtype=torch.uint8, device=q.device)
+        keep.append(ws)
+        P.workspace, P.workspace_bytes = _ptr(ws), ws.numel()
     rc = _lib.load().dsx_attn_fwd(P, _stream())
     _lib.check(rc, "dsx_attn_fwd")
     return (out, out2) if q2 is not None else out

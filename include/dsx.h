@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define DSX_ABI_VERSION 1
+#define DSX_ABI_VERSION 2
 
 enum {
   DSX_OK = 0,
@@ -171,6 +171,12 @@ typedef struct dsx_attn_params {
   const void* k_norm_w[2];
   float norm_eps;
   int32_t reserved;
+  /* Optional scratch for the fused pre-processing, owned by the caller (NULL = none): when it holds at
+   * least 2*batch*heads*(Sq+Skv)*128 bytes, q and k are normalised/rotated ONCE into it by a row kernel
+   * and the attention kernel reads them from there; without it the same arithmetic is applied inside the
+   * attention kernel as tiles are loaded, where every query block repeats the work on K. */
+  void* workspace;
+  int64_t workspace_bytes;
 } dsx_attn_params;
 
 int dsx_attn_fwd(const dsx_attn_params* p, void* stream);

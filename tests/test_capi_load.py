@@ -32,7 +32,7 @@ def test_abi_version_and_strerror():
     from diffsynth_engine_amd import _lib
 
     lib = _lib.load()
-    assert lib.dsx_abi_version() == 1
+    assert lib.dsx_abi_version() == 2
     assert _lib.strerror(0) == "ok"
     for code in (-1, -2, -3, -4, -5):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
@@ -43,8 +43,8 @@ def test_attn_params_struct_layout_matches_header():
     from diffsynth_engine_amd import _lib
 
     # 8 + 4 pointers/int64 pairs (12*8*... ) : q,k,v,o,sq,skv = 6*16; 12 strides*8; 3 int32 + float; rope, rope_sb;
-    # 2*16 norm pointers; float + int32
-    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 32 + 8
+    # 2*16 norm pointers; float + int32; workspace pointer + byte count
+    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 32 + 8 + 16
 
 
 def test_null_and_shape_errors_without_touching_the_gpu():

@@ -93,9 +93,11 @@ def _flux_ids(St, side):
     return torch.cat([txt, img.reshape(1, -1, 3)], dim=1)
 
 
+@pytest.mark.parametrize("in_kernel", [True, False])
 @pytest.mark.parametrize("wstd", [0.0, 0.1])
-def test_fused_rmsnorm_rope_joint_attention(dev, wstd):
-    """RMSNorm + 3-axis RoPE applied in-kernel == oracle RMSNorm -> concat -> apply_rope -> SDPA (flux_dit.py:161-183)."""
+def test_fused_rmsnorm_rope_joint_attention(dev, wstd, in_kernel):
+    """RMSNorm + 3-axis RoPE applied by the attention entry point (inside the kernel's tile loads, or once into
+    caller scratch) == oracle RMSNorm -> concat -> apply_rope -> SDPA (flux_dit.py:161-183)."""
     from diffsynth_engine_amd import ops
 
     H, St, side = 2, 64, 12
@@ -113,7 +115,7 @@ def test_fused_rmsnorm_rope_joint_attention(dev, wstd):
     table = ops.rope_table_from_freqs(freqs).to(dev)
     o1, o2 = ops.attention_bhsd(qt.to(dev), kt.to(dev), vt.to(dev), q2=qi.to(dev), k2=ki.to(dev), v2=vi.to(dev),
                                 rope=table, q_norm_w=w[2].to(dev), k_norm_w=w[3].to(dev), q2_norm_w=w[0].to(dev),
-                                k2_norm_w=w[1].to(dev))
+                                k2_norm_w=w[1].to(dev), in_kernel=in_kernel)
     got = torch.cat([o1.cpu(), o2.cpu()], dim=2)
     assert _rel_err(got, want) <= TOL
     # the standalone pre-pass must agree with the oracle's bf16 q almost bit for bit
