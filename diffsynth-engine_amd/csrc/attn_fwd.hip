@@ -465,7 +465,7 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
       (rc = check_seg(p->v, p->skv)) || (rc = check_seg((const void* const*)p->o, p->sq)))
     return rc;
   const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
-  if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 31) || Skv > (1ll << 31)) return DSX_EBADSHAPE;
+  if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 30) || Skv > (1ll << 30)) return DSX_EBADSHAPE;
   for (int g = 0; g < 2; ++g) {
     const int64_t strides[12] = {p->q_sb[g], p->q_sh[g], p->q_ss[g], p->k_sb[g], p->k_sh[g], p->k_ss[g],
                                  p->v_sb[g], p->v_sh[g], p->v_ss[g], p->o_sb[g], p->o_sh[g], p->o_ss[g]};

@@ -106,12 +106,17 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       vp[i] = vbase[seg] + lrow * p.v_ss[seg] * 2 + ((ld_p ^ ((row & 3) << 2)) << 4);
     }
   };
+  // uniform per-block pointer strides (bytes) of both segments, and the key counts as 32-bit scalars (the
+  // host bounds the sequence lengths), so that the per-interval bookkeeping is a few scalar instructions
+  const int skv0 = (int)p.skv[0], skv_all = (int)Skv;
+  const int64_t kstep[2] = {p.k_ss[0] * (2 * KB), p.k_ss[1] * (2 * KB)};
+  const int64_t vstep[2] = {p.v_ss[0] * (2 * KB), p.v_ss[1] * (2 * KB)};
   auto advance_to = [&](int kb) {  // called with consecutive kb
-    const int64_t k0 = (int64_t)kb * KB;
-    const int lo = k0 >= p.skv[0] ? 1 : 0, hi = k0 + KB - 1 >= p.skv[0] ? 1 : 0;
-    const bool simple = lo == hi && k0 + KB <= Skv;
+    const int k0 = kb * KB;
+    const int lo = k0 >= skv0 ? 1 : 0, hi = k0 + KB - 1 >= skv0 ? 1 : 0;
+    const bool simple = lo == hi && k0 + KB <= skv_all;
     if (simple && ptr_seg == lo) {
-      const int64_t ks = p.k_ss[lo] * (2 * KB), vs = p.v_ss[lo] * (2 * KB);
+      const int64_t ks = lo ? kstep[1] : kstep[0], vs = lo ? vstep[1] : vstep[0];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         kp[i] += ks;
@@ -122,16 +127,34 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
     }
     ptr_seg = simple ? lo : -1;
   };
-  auto issue_block = [&](int stage) {
-    uint8_t* sK = smem + stage * kTile + wave_u * 2048;
-    uint8_t* sV = sK + kStages * kTile;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      __builtin_amdgcn_global_load_lds((gptr_t)kp[i], (lptr_t)(sK + i * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)vp[i], (lptr_t)(sV + i * 1024), 16, 0, 0);
-    }
+  // The async loads are written as inline assembly on purpose: for a compiler-visible LDS-DMA the
+  // compiler cannot tell that the transposing LDS reads below never touch a stage that is still being
+  // filled, and puts s_waitcnt vmcnt(0) in front of them, which drains the whole prefetch pipeline in
+  // every interval.  Ordering against the reads is kept by hand: vmcnt waits + workgroup barriers.
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;
+  // (M0 carries the LDS destination; nothing else in this kernel uses M0)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+  auto dma16 = [&](const uint8_t* src, uint32_t lds_addr) {  // 64 lanes x 16 B -> lds_addr + lane*16
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(src), "s"(lds_addr)
+                 : "memory", "m0");
   };
-
+#pragma clang diagnostic pop
+  // one 1 KiB piece of the block the pointers address: which = 0, 1 -> K rows, 2, 3 -> V rows
+  auto issue_piece = [&](int stage, int which) {
+    const uint32_t sK = lds0 + stage * kTile + wave_u * 2048;
+    const uint32_t sV = sK + kStages * kTile;
+    if (which < 2)
+      dma16(kp[which], sK + which * 1024);
+    else
+      dma16(vp[which - 2], sV + (which - 2) * 1024);
+  };
+  auto issue_block = [&](int stage) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) issue_piece(stage, w);
+  };
   const int nkb = (int)((Skv + KB - 1) / KB);
   advance_to(0);
   issue_block(0);
@@ -187,31 +210,36 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
     lane_v[dt] = kStages * kTile + tr_key * 256 + ((dt ^ (tr_key & 3)) << 6) + tr_dbyte;
 
   // Software pipeline over 64-key blocks.  Interval kb (behind one workgroup barrier) runs
-  //   stage 1:  S(kb+1)^T = K(kb+1) Q^T on the matrix pipe, interleaved instruction by instruction
-  //             with P(kb) = exp2(S(kb)) -> bf16 and its row sums on the VALU (same wave, independent
-  //             registers: the MFMAs execute while the wave issues the exp2 / convert / dot work);
-  //   stage 2:  O^T += V(kb)^T P(kb)^T on the matrix pipe, then the block maximum of S(kb+1) and, when
-  //             it must move, the rescale of the softmax reference (VALU under the tail of the MFMAs).
-  // Without this a wave alternates MFMA-only and VALU-only phases, the two waves of a SIMD do so
-  // in step (they leave the barrier together), and the matrix pipe idles through every softmax.
+  //   stage 1:  S(kb+1)^T = K(kb+1) Q^T, 16 MFMAs;
+  //   stage 2:  O^T += V(kb)^T P(kb)^T, 16 MFMAs;
+  // and the softmax of the wave's own scores is spread over the 32 MFMA slots so that neither stage asks
+  // more of the VALU than the matrix pipe leaves time for when two waves share a SIMD: entries
+  // kExpEarly.. of P(kb) = exp2(S(kb)) in stage 1, the block maximum of S(kb+1) in the first slots of
+  // stage 2 (the PV MFMAs issued there cover the latency of the last QK MFMA), entries 0..kExpEarly-1 of
+  // P(kb+1) in the rest of stage 2.  The MFMAs execute while the wave issues the exp2 / convert / add
+  // work on independent registers.  Without this a wave alternates MFMA-only and VALU-only phases, the
+  // two waves of a SIMD do so in step (they leave the barrier together), and the matrix pipe idles
+  // through every softmax.
   // Four stages of K and V: block kb+1 must have landed when interval kb starts, kb+2 is in flight,
   // kb+3 is issued into the stage block kb-1 has left.
-  auto interval_head = [&](int kb, int load_stage) {
+  constexpr int kExpEarly = 12;  // even; entries of P(kb+1) produced during stage 2 of interval kb
+  constexpr int kAhead = 2;      // operand fragments in flight ahead of the MFMA that uses them
+  auto interval_head = [&](int kb) {
     __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4): only block kb+2 may still be in flight
     __builtin_amdgcn_s_barrier();
     if (kb + 3 < nkb) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
-    issue_block(load_stage);
   };
-  // softmax reference update for block `blk` whose scores are in s: masks the ragged tail, subtracts
-  // the current reference, and moves it (rescaling O and l) only when the block maximum demands it
-  auto ref_update = [&](f32x16 (&s)[2], int blk) {
-    if ((int64_t)(blk + 1) * KB > Skv) {  // ragged tail of the key axis
+  // Softmax reference.  ref_scan masks the ragged tail of block `blk`, subtracts the current reference and
+  // returns the block maximum of the lane's query; ref_move shifts the reference (rescaling O and l), which
+  // is needed only when a block maximum leaves the safe range.
+  auto ref_scan = [&](f32x16 (&s)[2], int blk) -> float {
+    if ((blk + 1) * KB > skv_all) {  // ragged tail of the key axis
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int64_t key = (int64_t)blk * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (key >= Skv) s[kt][r] = -INFINITY;
+          const int key = blk * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (key >= skv_all) s[kt][r] = -INFINITY;
         }
     }
     if (any_ref) {
@@ -227,22 +255,41 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       m0 = max3(m0, s[0][r], s[0][r + 1]);
       m1 = max3(m1, s[1][r], s[1][r + 1]);
     }
-    const float mx = pair_max(max3(m0, m1, fmaxf(s[0][15], s[1][15])));
+    return pair_max(max3(m0, m1, fmaxf(s[0][15], s[1][15])));
+  };
+  auto ref_must_move = [&](float mx, int blk) -> bool {  // wave-uniform
     const bool move = mx > kRescaleThreshold || (blk == 0 && mx < -kRescaleThreshold);
-    if (__builtin_amdgcn_ballot_w64(move) != 0) {
-      any_ref = true;
-      const float d = blk == 0 ? mx : fmaxf(mx, 0.f);
-      const float alpha = blk == 0 ? 1.0f : __builtin_amdgcn_exp2f(-d);
+    return __builtin_amdgcn_ballot_w64(move) != 0;
+  };
+  auto ref_move = [&](f32x16 (&s)[2], float mx, int blk) -> float {
+    any_ref = true;
+    const float d = blk == 0 ? mx : fmaxf(mx, 0.f);
+    const float alpha = blk == 0 ? 1.0f : __builtin_amdgcn_exp2f(-d);
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[kt][r] -= d;
-      m_ref += d;
-      l_run *= alpha;
+      for (int r = 0; r < 16; ++r) s[kt][r] -= d;
+    m_ref += d;
+    l_run *= alpha;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+      for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    return alpha;
+  };
+  // entry e (0..31) of P = exp2(S'): score s[e/16][e%16]; two entries pack into one bf16x2 word of the PV
+  // operand.  The row sum adds the fp32 values with plain v_add_f32 (v_dot2c_f32_bf16 on the packed pair
+  // would be one instruction, but it executes on the matrix pipe and was measured to cost a third of the
+  // MFMA rate).
+  float p_even = 0.f, lsum0 = 0.f, lsum1 = 0.f;
+  auto exp_entry = [&](const f32x16 (&s)[2], uint32_t (&pw)[2][8], int e) {
+    const float pv = __builtin_amdgcn_exp2f(s[e >> 4][e & 15]);
+    if (e & 1) {
+      pw[e >> 4][(e & 15) >> 1] = pack_bf16x2(p_even, pv);
+      lsum1 += pv;
+    } else {
+      p_even = pv;
+      lsum0 += pv;
     }
   };
   auto qk = [&](f32x16 (&s)[2], int stage) {
@@ -256,41 +303,24 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       }
     }
   };
-  // one interval; `stage` (= kb % 4) is a literal so that every LDS offset folds into an immediate
-  auto interval = [&](int kb, int stage, f32x16 (&s_cur)[2], f32x16 (&s_next)[2]) {
-    interval_head(kb, (stage + 3) % kStages);
-    // ---- stage 1: 16 slots, each = [LDS read of the K fragment two MFMAs ahead, one MFMA of
-    //      S(kb+1), two exp2 + one convert + one row-sum step of P(kb)]; sched_barrier pins the order
+  typedef short v8i16 __attribute__((ext_vector_type(8)));
+  // one interval; `stage` (= kb % 4) is a literal so that every LDS offset folds into an immediate.
+  // pw_cur holds entries 0..kExpEarly-1 of P(kb) on entry; pw_next holds those of P(kb+1) on exit.
+  auto interval = [&](int kb, int stage, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], uint32_t (&pw_cur)[2][8],
+                      uint32_t (&pw_next)[2][8]) {
+    interval_head(kb);
+    // The next block's four 1 KiB pieces go out between the MFMAs, K in stage 1 and V in stage 2: the CU's
+    // one address path takes ~25 cycles per piece, and a wave whose load queues behind the other waves'
+    // loads cannot issue its MFMAs meanwhile (32 pieces at once right after the barrier cost every wave
+    // 500-800 cycles).
+    constexpr int kLoadSlots[4] = {3, 11, 7, 13};
+    // ---- stage 1: 16 slots, each = [LDS read of the K fragment two MFMAs ahead, one MFMA of S(kb+1),
+    //      one or two entries of P(kb)]; sched_barrier pins the order
     const uint8_t* sK = smem + ((stage + 1) % kStages) * kTile;
     auto k_frag = [&](int i) {  // MFMA i of the block: k-chunk i/2, key tile i%2
       return *reinterpret_cast<const bf16x8*>(sK + lane_k[i >> 1] + (i & 1) * 8192);
     };
-    uint32_t pw[2][8];  // P as packed bf16, [kt][word]: entries 2w, 2w+1
-    float lsum0 = 0.f, lsum1 = 0.f;
-    bf16x8 kf[3];
-    kf[0] = k_frag(0);
-    kf[1] = k_frag(1);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if (i + 2 < 16) kf[(i + 2) % 3] = k_frag(i + 2);
-      const int kt = i & 1;
-      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % 3], qf[i >> 1], i < 2 ? zero16 : s_next[kt], 0, 0, 0);
-      // P = exp2(S'), packed to bf16 for the PV product; the row sum adds the fp32 values with plain
-      // v_add_f32 (v_dot2c_f32_bf16 on the packed pair would be one instruction, but it executes on the
-      // matrix pipe and was measured to cost a third of the MFMA rate)
-      const int pk = i >> 3, w = i & 7;
-      const float p0 = __builtin_amdgcn_exp2f(s_cur[pk][2 * w]);
-      const float p1 = __builtin_amdgcn_exp2f(s_cur[pk][2 * w + 1]);
-      pw[pk][w] = pack_bf16x2(p0, p1);
-      lsum0 += p0;
-      lsum1 += p1;
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    l_run += lsum0 + lsum1;
-    // ---- stage 2: O^T += V^T P^T, 16 slots = [transposing LDS reads of the V^T operand two MFMAs
-    //      ahead, one MFMA].  16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
     const uint8_t* sV = smem + stage * kTile;  // lane_v carries the offset of the V region
-    typedef short v8i16 __attribute__((ext_vector_type(8)));
     auto v_frag = [&](int j) {  // MFMA j: 16-key chunk j/4 (kt = j/8, ch = (j/4)%2), d tile j%4
       const uint8_t* src = sV + lane_v[j & 3] + (j >> 2) * 16 * 256;
       const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)src);
@@ -299,30 +329,89 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       const v8i16 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       return __builtin_bit_cast(bf16x8, both);
     };
-    bf16x8 vf[3];
-    vf[0] = v_frag(0);
-    vf[1] = v_frag(1);
+    // operand fragments are read kAhead MFMAs before their use; the last slots of stage 1 already fetch
+    // the first V^T fragments of stage 2 (block kb landed long ago), so only stage 1 starts cold
+    constexpr int kLate = 32 - kExpEarly;  // entries left for stage 1; the first kLate-16 slots take two
+    bf16x8 kf[kAhead + 1], vf[kAhead + 1];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      if (j + 2 < 16) vf[(j + 2) % 3] = v_frag(j + 2);
-      const int kt = j >> 3, ch = (j >> 2) & 1, dt = j & 3;
-      const u32x4 w = {pw[kt][4 * ch + 0], pw[kt][4 * ch + 1], pw[kt][4 * ch + 2], pw[kt][4 * ch + 3]};
-      oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[j % 3], __builtin_bit_cast(bf16x8, w), oacc[dt], 0, 0, 0);
+    for (int i = 0; i < kAhead; ++i) kf[i] = k_frag(i);
+    int e = kExpEarly;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (i + kAhead < 16)
+        kf[(i + kAhead) % (kAhead + 1)] = k_frag(i + kAhead);
+      else
+        vf[(i + kAhead - 16) % (kAhead + 1)] = v_frag(i + kAhead - 16);
+      const int kt = i & 1;
+      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % (kAhead + 1)], qf[i >> 1], i < 2 ? zero16 : s_next[kt], 0, 0, 0);
+      exp_entry(s_cur, pw_cur, e++);
+      if (i < kLate - 16) exp_entry(s_cur, pw_cur, e++);
+      if (i == kLoadSlots[0]) issue_piece((stage + 3) % kStages, 0);
+      if (i == kLoadSlots[1]) issue_piece((stage + 3) % kStages, 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (kb + 1 < nkb) ref_update(s_next, kb + 1);
+    l_run += lsum0 + lsum1;
+    lsum0 = lsum1 = 0.f;
+    // ---- stage 2: O^T += V^T P^T, 16 slots = [transposing LDS reads of a V^T operand, one MFMA].
+    //      16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
+    auto pv_slot = [&](int j) {
+      if (j + kAhead < 16) vf[(j + kAhead) % (kAhead + 1)] = v_frag(j + kAhead);
+      const int kt = j >> 3, ch = (j >> 2) & 1, dt = j & 3;
+      const u32x4 w = {pw_cur[kt][4 * ch + 0], pw_cur[kt][4 * ch + 1], pw_cur[kt][4 * ch + 2], pw_cur[kt][4 * ch + 3]};
+      oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[j % (kAhead + 1)], __builtin_bit_cast(bf16x8, w), oacc[dt], 0, 0, 0);
+    };
+    constexpr int kScanSlots = 4;  // PV MFMAs issued before the block maximum of S(kb+1) is looked at
+#pragma unroll
+    for (int j = 0; j < kScanSlots; ++j) {
+      pv_slot(j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kb + 1 < nkb) {
+      const float mx = ref_scan(s_next, kb + 1);
+      if (ref_must_move(mx, kb + 1)) {
+        // rare: O, l and the scores of block kb+1 move to the new reference now; the part of P(kb) that
+        // the remaining PV MFMAs still have to accumulate follows (one more bf16 rounding on it)
+        const float alpha = ref_move(s_next, mx, kb + 1);
+#pragma unroll
+        for (int j = kScanSlots; j < 16; j += 4)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            uint32_t& word = pw_cur[j >> 3][4 * ((j >> 2) & 1) + w];
+            word = pack_bf16x2(bf16_lo(word) * alpha, bf16_hi(word) * alpha);
+          }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // (in the last interval the entries below come from a block that does not exist and are dropped)
+    int e2 = 0;
+#pragma unroll
+    for (int j = kScanSlots; j < 16; ++j) {
+      pv_slot(j);
+      // kExpEarly entries over the 16 - kScanSlots remaining slots, the surplus in the first ones
+      exp_entry(s_next, pw_next, e2++);
+      if (j - kScanSlots < kExpEarly - (16 - kScanSlots)) exp_entry(s_next, pw_next, e2++);
+      if (j == kLoadSlots[2]) issue_piece((stage + 3) % kStages, 2);
+      if (j == kLoadSlots[3]) issue_piece((stage + 3) % kStages, 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   f32x16 sA[2], sB[2];
+  uint32_t pwA[2][8], pwB[2][8];
   __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): block 0 has landed
   __builtin_amdgcn_s_barrier();
   qk(sA, 0);
-  ref_update(sA, 0);
+  {
+    const float mx = ref_scan(sA, 0);
+    if (ref_must_move(mx, 0)) ref_move(sA, mx, 0);
+#pragma unroll
+    for (int e = 0; e < kExpEarly; ++e) exp_entry(sA, pwA, e);
+  }
   for (int kb = 0; kb < nkb; kb += 4) {
-    interval(kb, 0, sA, sB);
-    if (kb + 1 < nkb) interval(kb + 1, 1, sB, sA);
-    if (kb + 2 < nkb) interval(kb + 2, 2, sA, sB);
-    if (kb + 3 < nkb) interval(kb + 3, 3, sB, sA);
+    interval(kb, 0, sA, sB, pwA, pwB);
+    if (kb + 1 < nkb) interval(kb + 1, 1, sB, sA, pwB, pwA);
+    if (kb + 2 < nkb) interval(kb + 2, 2, sA, sB, pwA, pwB);
+    if (kb + 3 < nkb) interval(kb + 3, 3, sB, sA, pwB, pwA);
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain trailing async loads
 
