@@ -44,7 +44,7 @@ class AttnParams(ctypes.Structure):
         ("q_norm_w", c_void_p * 2),
         ("k_norm_w", c_void_p * 2),
         ("norm_eps", c_float),
-        ("reserved", ctypes.c_int32),
+        ("score_bound", ctypes.c_float),
         ("workspace", c_void_p),
         ("workspace_bytes", c_int64),
     ]

@@ -54,6 +54,9 @@ __device__ __forceinline__ float pair_sum(float v) {
 }
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
+// SCAN = false: the caller has bounded every |score| (log2 domain) by kRescaleThreshold, so the softmax
+// reference can stay 0 for the whole row and the per-block maximum is not computed at all.
+template <bool SCAN>
 __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x;
@@ -229,10 +232,10 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
     __builtin_amdgcn_s_barrier();
     if (kb + 3 < nkb) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
   };
-  // Softmax reference.  ref_scan masks the ragged tail of block `blk`, subtracts the current reference and
-  // returns the block maximum of the lane's query; ref_move shifts the reference (rescaling O and l), which
+  // Softmax reference.  mask_tail masks the ragged tail of block `blk`; ref_scan subtracts the current
+  // reference and returns the block maximum of the lane's query; ref_move shifts the reference (rescaling O and l), which
   // is needed only when a block maximum leaves the safe range.
-  auto ref_scan = [&](f32x16 (&s)[2], int blk) -> float {
+  auto mask_tail = [&](f32x16 (&s)[2], int blk) {
     if ((blk + 1) * KB > skv_all) {  // ragged tail of the key axis
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -242,6 +245,8 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
           if (key >= skv_all) s[kt][r] = -INFINITY;
         }
     }
+  };
+  auto ref_scan = [&](f32x16 (&s)[2], int blk) -> float {
     if (any_ref) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -367,8 +372,9 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     if (kb + 1 < nkb) {
-      const float mx = ref_scan(s_next, kb + 1);
-      if (ref_must_move(mx, kb + 1)) {
+      mask_tail(s_next, kb + 1);
+      const float mx = SCAN ? ref_scan(s_next, kb + 1) : 0.f;
+      if (SCAN && ref_must_move(mx, kb + 1)) {
         // rare: O, l and the scores of block kb+1 move to the new reference now; the part of P(kb) that
         // the remaining PV MFMAs still have to accumulate follows (one more bf16 rounding on it)
         const float alpha = ref_move(s_next, mx, kb + 1);
@@ -402,8 +408,11 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   __builtin_amdgcn_s_barrier();
   qk(sA, 0);
   {
-    const float mx = ref_scan(sA, 0);
-    if (ref_must_move(mx, 0)) ref_move(sA, mx, 0);
+    mask_tail(sA, 0);
+    if (SCAN) {
+      const float mx = ref_scan(sA, 0);
+      if (ref_must_move(mx, 0)) ref_move(sA, mx, 0);
+    }
 #pragma unroll
     for (int e = 0; e < kExpEarly; ++e) exp_entry(sA, pwA, e);
   }
@@ -439,7 +448,9 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
 int launch_attn_plain(const dsx_attn_params& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)attn_plain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)attn_plain_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)attn_plain_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             kLdsBytes) != hipSuccess)
       return DSX_ELAUNCH;
     attr_set = true;
@@ -448,7 +459,13 @@ int launch_attn_plain(const dsx_attn_params& p, hipStream_t st) {
   const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
   if (units > (1ll << 30)) return DSX_EBADSHAPE;
   dim3 grid((unsigned)(((units + 7) / 8) * 8)), block(512);
-  attn_plain_kernel<<<grid, block, kLdsBytes, st>>>(p);
+  // a caller-supplied bound on |softmax_scale * q.k| that keeps exp2 of every score inside fp32 and bf16
+  // with a fixed reference lets the kernel skip the per-block maximum
+  const bool bounded = p.score_bound > 0.f && p.score_bound * kLog2e <= kRescaleThreshold;
+  if (bounded)
+    attn_plain_kernel<false><<<grid, block, kLdsBytes, st>>>(p);
+  else
+    attn_plain_kernel<true><<<grid, block, kLdsBytes, st>>>(p);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 

@@ -116,6 +116,20 @@ class FluxDiTRunner:
             elif key.endswith(".bias"):
                 self.lin[key[: -len(".bias")]].b = t.to(self.device, torch.bfloat16).contiguous()
         self.has_guidance = "guidance_embedder.timestep_embedder.0" in self.lin
+        # After RMSNorm over the head dim every q and k row has norm <= sqrt(128) * max|weight| and RoPE keeps
+        # norms, so |q.k| / sqrt(128) <= sqrt(128) * max|w_q| * max|w_k|: the attention kernel is told so and
+        # drops its running maximum where that keeps exp2 in range (2 % slack for the bf16 roundings).
+        self.score_bound: Dict[str, float] = {}
+        wmax = {k: float(v.float().abs().max()) for k, v in self.norm_w.items()}
+        for i in range(num_double):
+            pre = f"blocks.{i}.attn."
+            if all(pre + n in wmax for n in ("norm_q_a", "norm_q_b", "norm_k_a", "norm_k_b")):
+                self.score_bound[f"blocks.{i}."] = 1.02 * math.sqrt(HEAD_DIM) * max(
+                    wmax[pre + "norm_q_a"], wmax[pre + "norm_q_b"]) * max(wmax[pre + "norm_k_a"], wmax[pre + "norm_k_b"])
+        for i in range(num_single):
+            pre = f"single_blocks.{i}."
+            if pre + "norm_q_a" in wmax and pre + "norm_k_a" in wmax:
+                self.score_bound[pre] = 1.02 * math.sqrt(HEAD_DIM) * wmax[pre + "norm_q_a"] * wmax[pre + "norm_k_a"]
         self._stack_modulation()
 
     def _stack_modulation(self):
@@ -222,7 +236,7 @@ class FluxDiTRunner:
                                out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2), in_kernel=True)
         else:
             ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2),
-                               out2=o_a.transpose(1, 2))
+                               out2=o_a.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
         # The two streams run the same sequence on different weights (flux_dit.py:226-234): out-projection +
         # gated residual, LN-modulate, MLP + gated residual.  Each pair of linears goes out as one grouped
         # submission so that the 512-token text problem runs beside the image problem instead of after it.
@@ -259,7 +273,7 @@ class FluxDiTRunner:
         else:
             ops.rmsnorm_rope_qk(h.view(B, S, 7 * d), HEADS, HEADS, nw[pre + "norm_q_a"], nw[pre + "norm_k_a"], rope,
                                 0, EPS)
-            ops.attention_bhsd(q_, k_, v_, out=att.transpose(1, 2))
+            ops.attention_bhsd(q_, k_, v_, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
         # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
         # parts and emits the e4m3 operand of proj_out with its per-token scale
         if self.scaled:

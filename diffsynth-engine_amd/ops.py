@@ -192,7 +192,7 @@ def rope_table_from_freqs(freqs: torch.Tensor) -> torch.Tensor:
 def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float] = None,
                    rope: Optional[torch.Tensor] = None, q_norm_w=None, k_norm_w=None, q2_norm_w=None,
                    k2_norm_w=None, eps: float = 1e-6, out: Optional[torch.Tensor] = None,
-                   out2: Optional[torch.Tensor] = None, in_kernel: bool = False):
+                   out2: Optional[torch.Tensor] = None, in_kernel: bool = False, score_bound: float = 0.0):
     """softmax(q k^T * scale) v over the concatenation [segment 1, segment 2] of rows.
 
     q, k, v: (B,H,S,128) bf16 views with unit stride in the last dim (any other strides).
@@ -201,6 +201,8 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     *_norm_w: optional (128,) bf16 RMSNorm weights applied before RoPE.
     in_kernel: apply RoPE / RMSNorm inside the attention kernel as tiles are loaded (every query block then
     repeats the work on K); default: normalise / rotate q and k once into a scratch buffer allocated here.
+    score_bound: optional promise |scale * q.k| <= score_bound for every pair (after RMSNorm/RoPE); when it is
+    small enough the kernel skips the running softmax maximum (same result).  0 = no promise.
     Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).
     """
     _require_cuda(q, k, v)
@@ -247,6 +249,7 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
                 keep.append(w)
                 getattr(P, name)[i] = _ptr(w)
     P.norm_eps = eps
+    P.score_bound = float(score_bound)
     if keep and not in_kernel:
         ws = torch.empty(2 * B * H * (S1 + S2 + Skv1 + Skv2) * D, dtype=torch.uint8, device=q.device)
         keep.append(ws)

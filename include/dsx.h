@@ -170,7 +170,12 @@ typedef struct dsx_attn_params {
   const void* q_norm_w[2];
   const void* k_norm_w[2];
   float norm_eps;
-  int32_t reserved;
+  /* Optional promise by the caller: |softmax_scale * q.k| <= score_bound for every query/key pair after
+   * the pre-processing above (0 = no promise).  With score_bound*log2(e) <= 64 the kernel keeps the
+   * softmax reference at 0 and skips the running maximum; the result is the same softmax.  E.g. after
+   * RMSNorm over head_dim with weights wq, wk: head_dim * max|wq| * max|wk| * softmax_scale.  A promise
+   * that does not hold can overflow exp2. */
+  float score_bound;
   /* Optional scratch for the fused pre-processing, owned by the caller (NULL = none): when it holds at
    * least 2*batch*heads*(Sq+Skv)*128 bytes, q and k are normalised/rotated ONCE into it by a row kernel
    * and the attention kernel reads them from there; without it the same arithmetic is applied inside the

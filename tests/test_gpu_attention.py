@@ -184,3 +184,25 @@ def test_rmsnorm_rope_qk_in_place_equals_per_tensor_kernel(dev, H, S, extra):
     diff = (got_h[:, :H].float() - ref.float()).abs()
     assert (diff > 0).float().mean().item() < 0.01
     assert diff.max().item() <= 2 ** -6 * ref.float().abs().max().item()
+
+
+@pytest.mark.parametrize("Sq,Skv", [(300, 300), (64, 1000), (257, 77)])
+def test_score_bound_promise_skips_the_running_maximum(dev, Sq, Skv):
+    """Rows of norm sqrt(128) (what q/k RMSNorm with unit weights produces) bound |q.k|/sqrt(128) by sqrt(128);
+    with that promise the kernel keeps its softmax reference at 0.  Same result as without the promise (on
+    such inputs neither variant ever moves the reference), and both match fp32 SDPA.  A promise too large to
+    be of use is ignored."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(Sq + Skv)
+    unit = lambda t: (t / t.norm(dim=-1, keepdim=True) * math.sqrt(128)).bfloat16()
+    q = unit(torch.randn(1, 3, Sq, 128, generator=g))
+    k = unit(torch.randn(1, 3, Skv, 128, generator=g))
+    k[0, 0, : min(Sq, Skv)] = q[0, 0, : min(Sq, Skv)]  # some scores right at the bound
+    v = torch.randn(1, 3, Skv, 128, generator=g).bfloat16()
+    want = O.sdpa(q.float(), k.float(), v.float())
+    plain = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev)).cpu()
+    bounded = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=1.02 * math.sqrt(128)).cpu()
+    ignored = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=1e4).cpu()
+    assert torch.equal(plain, bounded) and torch.equal(plain, ignored)
+    assert _rel_err(bounded, want) <= TOL
