@@ -80,15 +80,37 @@ __device__ __forceinline__ float e4m3_bits_to_f32(uint32_t b) {
   return __uint_as_float(__float_as_uint(v) | sign);
 }
 
+// Wavefront-wide butterfly reductions (every lane ends with the result).  Steps 32 and 16 use the gfx950
+// lane-swap instructions, steps 8..1 fold a DPP row rotate / quad permute into the add or max itself: six
+// short VALU instructions instead of six trips through the LDS crossbar (ds_bpermute).  Same pairing, same
+// order (32, 16, 8, 4, 2, 1) and therefore the same fp32 result as the xor butterfly.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppRowRor8 = 0x128, kDppRowRor4 = 0x124, kDppQuadXor2 = 0x4e, kDppQuadXor1 = 0xb1;
+
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+  v = fmaxf(v, dpp_f32<kDppRowRor8>(v));
+  v = fmaxf(v, dpp_f32<kDppRowRor4>(v));
+  v = fmaxf(v, dpp_f32<kDppQuadXor2>(v));
+  v = fmaxf(v, dpp_f32<kDppQuadXor1>(v));
   return v;
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(b[0]) + __uint_as_float(b[1]);
+  v += dpp_f32<kDppRowRor8>(v);
+  v += dpp_f32<kDppRowRor4>(v);
+  v += dpp_f32<kDppQuadXor2>(v);
+  v += dpp_f32<kDppQuadXor1>(v);
   return v;
 }
 

@@ -214,27 +214,56 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
   __builtin_amdgcn_wave_barrier();
   const int ch = lane & 15, r0 = lane >> 4;
   const int n = n_base + ch * 8;
+  const bool col_ok = n < p.N;
+  // The gate is one vector per batch element: when the wave's 128 rows lie in one batch element (always,
+  // unless a tile straddles two) it is fetched once, and the row -> batch division leaves the row loop.
+  u32x4 gv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  bool gate_per_row = false;
+  const bool gated = RESID && p.gate != nullptr;
+  if (gated) {
+    const int b_lo = m_base / p.rows_per_batch, b_hi = min(m_base + 127, p.M - 1) / p.rows_per_batch;
+    gate_per_row = b_lo != b_hi;
+    if (!gate_per_row && col_ok) gv = *reinterpret_cast<const u32x4*>(p.gate + (int64_t)b_lo * p.gate_sb + n);
+  }
+  // rows are handled eight at a time so that the residual loads of a group are in flight together;
+  // interior tiles (the common case) run without per-row bounds tests
+  auto rows8 = [&](int it0, bool guarded) {
+    u32x4 v[8], rv[8];
+    bool ok[8];
 #pragma unroll
-  for (int it = 0; it < 32; ++it) {
-    const int ml = it * 4 + r0;
-    u32x4 v = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
-    const int m = m_base + ml;
-    if (m < p.M && n < p.N) {
+    for (int u = 0; u < 8; ++u) {
+      const int ml = (it0 + u) * 4 + r0;
+      const int m = m_base + ml;
+      ok[u] = !guarded || (m < p.M && col_ok);
+      v[u] = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
+      if (RESID && ok[u]) rv[u] = *reinterpret_cast<const u32x4*>(p.resid + (int64_t)m * p.ldr + n);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int m = m_base + (it0 + u) * 4 + r0;
+      if (!ok[u]) continue;
       if (RESID) {
+        u32x4 gu = gv;
+        if (gate_per_row)
+          gu = *reinterpret_cast<const u32x4*>(p.gate + (int64_t)(m / p.rows_per_batch) * p.gate_sb + n);
         // rounding points of the separate ops: bf16(gate * proj), then bf16(resid + .)
-        const u32x4 rv = *reinterpret_cast<const u32x4*>(p.resid + (int64_t)m * p.ldr + n);
-        u32x4 gv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
-        if (p.gate)
-          gv = *reinterpret_cast<const u32x4*>(p.gate + (int64_t)(m / p.rows_per_batch) * p.gate_sb + n);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float t0 = p.gate ? round_bf16(bf16_lo(gv[e]) * bf16_lo(v[e])) : bf16_lo(v[e]);
-          const float t1 = p.gate ? round_bf16(bf16_hi(gv[e]) * bf16_hi(v[e])) : bf16_hi(v[e]);
-          v[e] = pack_bf16x2(bf16_lo(rv[e]) + t0, bf16_hi(rv[e]) + t1);
+        for (int c = 0; c < 4; ++c) {
+          const float t0 = gated ? round_bf16(bf16_lo(gu[c]) * bf16_lo(v[u][c])) : bf16_lo(v[u][c]);
+          const float t1 = gated ? round_bf16(bf16_hi(gu[c]) * bf16_hi(v[u][c])) : bf16_hi(v[u][c]);
+          v[u][c] = pack_bf16x2(bf16_lo(rv[u][c]) + t0, bf16_hi(rv[u][c]) + t1);
         }
       }
-      *reinterpret_cast<u32x4*>(p.out + (int64_t)m * p.ldo + n) = v;
+      *reinterpret_cast<u32x4*>(p.out + (int64_t)m * p.ldo + n) = v[u];
     }
+  };
+  const bool interior = m_base + 128 <= p.M && n_base + 128 <= p.N;  // wave-uniform
+  if (interior) {
+#pragma unroll
+    for (int it0 = 0; it0 < 32; it0 += 8) rows8(it0, false);
+  } else {
+#pragma unroll
+    for (int it0 = 0; it0 < 32; it0 += 8) rows8(it0, true);
   }
 }
 
