@@ -88,6 +88,7 @@ SIGNATURES = {
     "dsx_concat_gelu_tanh": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
                                      c_int64, c_void_p, c_int64, c_int64, c_void_p]),
     "dsx_attn_fwd": (c_int, [ctypes.POINTER(AttnParams), c_void_p]),
+    "dsx_attn_workspace_bytes": (c_int64, [ctypes.POINTER(AttnParams)]),
     "dsx_rmsnorm_rope": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int64,
                                  c_int64, c_void_p, c_int64, c_int64, c_int64, ctypes.c_int32, ctypes.c_int32,
                                  c_int64, c_void_p]),

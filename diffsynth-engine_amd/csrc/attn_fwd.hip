@@ -479,12 +479,12 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
   for (int g = 0; g < 2; ++g)
     if (((uintptr_t)p->q_norm_w[g] & 15) || ((uintptr_t)p->k_norm_w[g] & 15)) return DSX_EALIGN;
 
-  if (!fused) return launch_attn_plain(*p, (hipStream_t)stream);
+  if (p->workspace && ((uintptr_t)p->workspace & 15)) return DSX_EALIGN;
+  if (!fused) return launch_attn_plain(*p, p->workspace, p->workspace ? p->workspace_bytes : 0, (hipStream_t)stream);
 
   // With caller scratch: normalise / rotate q and k once into it, then run the plain kernel on the copies.
   const int64_t ws_need = 2 * (int64_t)p->batch * p->heads * (Sq + Skv) * HD;
   if (p->workspace && p->workspace_bytes >= ws_need) {
-    if ((uintptr_t)p->workspace & 15) return DSX_EALIGN;
     hipStream_t st = (hipStream_t)stream;
     dsx_attn_params t = *p;
     uint16_t* wq = (uint16_t*)p->workspace;
@@ -519,7 +519,8 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
     if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
     t.rope = nullptr;
     t.q_norm_w[0] = t.q_norm_w[1] = t.k_norm_w[0] = t.k_norm_w[1] = nullptr;
-    return launch_attn_plain(t, st);
+    // what the copies leave of the scratch serves the key-range split of the attention kernel
+    return launch_attn_plain(t, (uint8_t*)p->workspace + ws_need, p->workspace_bytes - ws_need, st);
   }
 
   static bool attr_set = false;
@@ -582,4 +583,14 @@ extern "C" int dsx_rmsnorm_rope_qk(void* x, int64_t x_sb, int64_t x_ss, int32_t 
       (uint16_t*)x, x_sb, x_ss, heads_q, heads_k, (const uint16_t*)q_norm_w, (const uint16_t*)k_norm_w, eps,
       rope, rope_sb, rope_pos0, seq);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}
+
+extern "C" int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p) {
+  using namespace dsx;
+  if (!p || p->head_dim != HD || p->batch <= 0 || p->heads <= 0) return 0;
+  const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
+  if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 30) || Skv > (1ll << 30)) return 0;
+  const bool fused = p->rope || p->q_norm_w[0] || p->q_norm_w[1] || p->k_norm_w[0] || p->k_norm_w[1];
+  const int64_t copies = fused ? 2 * (int64_t)p->batch * p->heads * (Sq + Skv) * HD : 0;
+  return copies + attn_plain_workspace_bytes(*p);
 }

@@ -54,10 +54,43 @@ __device__ __forceinline__ float pair_sum(float v) {
 }
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
+// Key-range split of the last, partly filled round of workgroups.  With U units on C compute units the
+// last round keeps only U mod C of them busy; instead, the first `full_units` units run whole (one
+// workgroup each) and the key axes of the remaining `tail_units` are laid end to end and cut into
+// `pieces` equal runs of `len` 64-key blocks, one workgroup each, so that the last round ends everywhere
+// at once.  A piece covers the end of one unit and/or the start of the next; each part leaves its
+// unnormalised O, row sums and softmax references in a slot, and attn_merge_kernel combines the parts
+// of a unit.
+struct AttnSplit {
+  int full_units, tail_units, pieces, len, max_parts;
+  float* slots;
+};
+constexpr int kSlotOFloats = QB * HD;               // O part: [dt][rq][wave][g][j][4]
+constexpr int kSlotFloats = kSlotOFloats + 2 * QB;  // + row sums, + references
+
+// normalised output of one lane: query `row`, d = dt*32 + 8*rq + 4g + 0..3 per (dt, rq)
+__device__ __forceinline__ void store_output(const dsx_attn_params& p, int b, int h, int64_t row, int g,
+                                             const f32x16 (&oacc)[4], float inv) {
+  const int seg = row >= p.sq[0] ? 1 : 0;
+  uint16_t* dst = (uint16_t*)p.o[seg] + (int64_t)b * p.o_sb[seg] + (int64_t)h * p.o_sh[seg] +
+                  (row - (seg ? p.sq[0] : 0)) * p.o_ss[seg];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      u32x2 w;
+      w.x = pack_bf16x2(oacc[dt][4 * rq + 0] * inv, oacc[dt][4 * rq + 1] * inv);
+      w.y = pack_bf16x2(oacc[dt][4 * rq + 2] * inv, oacc[dt][4 * rq + 3] * inv);
+      *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w;
+    }
+}
+
 // SCAN = false: the caller has bounded every |score| (log2 domain) by kRescaleThreshold, so the softmax
 // reference can stay 0 for the whole row and the per-block maximum is not computed at all.
-template <bool SCAN>
-__global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
+// SPLIT = false: every workgroup runs one whole unit (sp.full_units = all of them); the loop over parts
+// and the variable key range fold away.
+template <bool SCAN, bool SPLIT>
+__global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, AttnSplit sp) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -67,14 +100,39 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   // query block) units so that the query blocks of one head share that head's K/V through ONE L2
   // (with a plain 3-D grid every XCD ends up fetching every head's K and V).
   const int nqb = (int)((p.sq[0] + p.sq[1] + QB - 1) / QB);
-  const int total_units = nqb * p.heads * p.batch;
-  const int unit = (int)(blockIdx.x & 7) * ((total_units + 7) >> 3) + (int)(blockIdx.x >> 3);
-  if (unit >= total_units) return;
-  const int qblk = unit % nqb;
-  const int h = (unit / nqb) % p.heads, b = unit / (nqb * p.heads);
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int64_t Skv = p.skv[0] + p.skv[1];
+  const int nkb = (int)((Skv + KB - 1) / KB);
+  // what this workgroup does: one whole unit, or one piece of the split tail = up to two parts of units
+  int nparts = 1, part_unit[2], part_kb0[2], part_kb1[2];
+  const int full8 = (sp.full_units + 7) & ~7;
+  if (!SPLIT || (int)blockIdx.x < full8) {
+    part_unit[0] = (int)(blockIdx.x & 7) * (full8 >> 3) + (int)(blockIdx.x >> 3);
+    if (part_unit[0] >= sp.full_units) return;
+    part_kb0[0] = 0;
+    part_kb1[0] = nkb;
+  } else {
+    const int piece = (int)blockIdx.x - full8;
+    const int it0 = piece * sp.len, it1 = min(it0 + sp.len, sp.tail_units * nkb);
+    if (piece >= sp.pieces || it0 >= it1) return;
+    const int t0 = it0 / nkb, t1 = (it1 - 1) / nkb;
+    part_unit[0] = sp.full_units + t0;
+    part_kb0[0] = it0 - t0 * nkb;
+    part_kb1[0] = t1 == t0 ? it1 - t0 * nkb : nkb;
+    if (t1 != t0) {
+      nparts = 2;
+      part_unit[1] = sp.full_units + t1;
+      part_kb0[1] = 0;
+      part_kb1[1] = it1 - t1 * nkb;
+    }
+  }
+  for (int part = 0; part < (SPLIT ? nparts : 1); ++part) {
+  const int unit = part_unit[part];
+  const int kb_begin = SPLIT ? part_kb0[part] : 0, kb_end = SPLIT ? part_kb1[part] : nkb;
+  const int qblk = unit % nqb;
+  const int h = (unit / nqb) % p.heads, b = unit / (nqb * p.heads);
   const int64_t q0 = (int64_t)qblk * QB + wave * 32;
+  if (SPLIT && part) __syncthreads();  // the stages of the previous part have been read for the last time
 
   const uint16_t* qbase[2];
   const uint8_t* kbase[2];
@@ -158,12 +216,11 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
 #pragma unroll
     for (int w = 0; w < 4; ++w) issue_piece(stage, w);
   };
-  const int nkb = (int)((Skv + KB - 1) / KB);
-  advance_to(0);
+  advance_to(kb_begin);
   issue_block(0);
-  if (nkb > 1) advance_to(1);
+  if (kb_begin + 1 < kb_end) advance_to(kb_begin + 1);
   issue_block(1);
-  if (nkb > 2) advance_to(2);
+  if (kb_begin + 2 < kb_end) advance_to(kb_begin + 2);
   issue_block(2);
 
   // ---- Q fragments (B operand of S^T = K Q^T), pre-multiplied by scale*log2(e)
@@ -230,7 +287,7 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   auto interval_head = [&](int kb) {
     __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4): only block kb+2 may still be in flight
     __builtin_amdgcn_s_barrier();
-    if (kb + 3 < nkb) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
+    if (kb + 3 < kb_end) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
   };
   // Softmax reference.  mask_tail masks the ragged tail of block `blk`; ref_scan subtracts the current
   // reference and returns the block maximum of the lane's query; ref_move shifts the reference (rescaling O and l), which
@@ -263,13 +320,13 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
     return pair_max(max3(m0, m1, fmaxf(s[0][15], s[1][15])));
   };
   auto ref_must_move = [&](float mx, int blk) -> bool {  // wave-uniform
-    const bool move = mx > kRescaleThreshold || (blk == 0 && mx < -kRescaleThreshold);
+    const bool move = mx > kRescaleThreshold || (blk == kb_begin && mx < -kRescaleThreshold);
     return __builtin_amdgcn_ballot_w64(move) != 0;
   };
   auto ref_move = [&](f32x16 (&s)[2], float mx, int blk) -> float {
     any_ref = true;
-    const float d = blk == 0 ? mx : fmaxf(mx, 0.f);
-    const float alpha = blk == 0 ? 1.0f : __builtin_amdgcn_exp2f(-d);
+    const float d = blk == kb_begin ? mx : fmaxf(mx, 0.f);
+    const float alpha = blk == kb_begin ? 1.0f : __builtin_amdgcn_exp2f(-d);
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -371,7 +428,7 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
       pv_slot(j);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (kb + 1 < nkb) {
+    if (kb + 1 < kb_end) {
       mask_tail(s_next, kb + 1);
       const float mx = SCAN ? ref_scan(s_next, kb + 1) : 0.f;
       if (SCAN && ref_must_move(mx, kb + 1)) {
@@ -408,65 +465,169 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p) {
   __builtin_amdgcn_s_barrier();
   qk(sA, 0);
   {
-    mask_tail(sA, 0);
+    mask_tail(sA, kb_begin);
     if (SCAN) {
-      const float mx = ref_scan(sA, 0);
-      if (ref_must_move(mx, 0)) ref_move(sA, mx, 0);
+      const float mx = ref_scan(sA, kb_begin);
+      if (ref_must_move(mx, kb_begin)) ref_move(sA, mx, kb_begin);
     }
 #pragma unroll
     for (int e = 0; e < kExpEarly; ++e) exp_entry(sA, pwA, e);
   }
-  for (int kb = 0; kb < nkb; kb += 4) {
+  for (int kb = kb_begin; kb < kb_end; kb += 4) {  // stage of block kb = (kb - kb_begin) % 4
     interval(kb, 0, sA, sB, pwA, pwB);
-    if (kb + 1 < nkb) interval(kb + 1, 1, sB, sA, pwB, pwA);
-    if (kb + 2 < nkb) interval(kb + 2, 2, sA, sB, pwA, pwB);
-    if (kb + 3 < nkb) interval(kb + 3, 3, sB, sA, pwB, pwA);
+    if (kb + 1 < kb_end) interval(kb + 1, 1, sB, sA, pwB, pwA);
+    if (kb + 2 < kb_end) interval(kb + 2, 2, sA, sB, pwA, pwB);
+    if (kb + 3 < kb_end) interval(kb + 3, 3, sB, sA, pwB, pwA);
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain trailing async loads
 
-  // ---- normalise and store.  lane (g, j): query j, d = dt*32 + 8*(r/4) + 4g + r%4
-  const float inv = 1.0f / pair_sum(l_run);
+  // ---- lane (g, j): query j, d = dt*32 + 8*(r/4) + 4g + r%4
+  const float l_row = pair_sum(l_run);
   const int64_t row = q0 + li;
-  if (row < Sq) {
-    const int seg = row >= p.sq[0] ? 1 : 0;
-    uint16_t* dst = (uint16_t*)p.o[seg] + (int64_t)b * p.o_sb[seg] + (int64_t)h * p.o_sh[seg] +
-                    (row - (seg ? p.sq[0] : 0)) * p.o_ss[seg];
+  if (!SPLIT || (kb_begin == 0 && kb_end == nkb)) {  // the whole key axis: normalise and store
+    if (row < Sq) store_output(p, b, h, row, g, oacc, 1.0f / l_row);
+  } else {                               // a part: leave O, l and the reference for the merge
+    const int t = unit - sp.full_units;
+    const int first_piece = (t * nkb) / sp.len;
+    const int my_piece = (t * nkb + kb_begin) / sp.len;
+    float* slot = sp.slots + (int64_t)(t * sp.max_parts + (my_piece - first_piece)) * kSlotFloats;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        u32x2 w;
-        w.x = pack_bf16x2(oacc[dt][4 * rq + 0] * inv, oacc[dt][4 * rq + 1] * inv);
-        w.y = pack_bf16x2(oacc[dt][4 * rq + 2] * inv, oacc[dt][4 * rq + 3] * inv);
-        *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w;
+        const f32x4 v = {oacc[dt][4 * rq + 0], oacc[dt][4 * rq + 1], oacc[dt][4 * rq + 2], oacc[dt][4 * rq + 3]};
+        *reinterpret_cast<f32x4*>(slot + ((((dt * 4 + rq) * 8 + wave) * 2 + g) * 32 + li) * 4) = v;
+      }
+    if (g == 0) {
+      slot[kSlotOFloats + wave * 32 + li] = l_row;
+      slot[kSlotOFloats + QB + wave * 32 + li] = m_ref;
+    }
+  }
+  }  // parts
+}
+
+// Combines the parts of every split unit: O = sum_i O_i 2^(m_i - m), l likewise, m = max_i m_i.
+// Same lane <-> (query, d) mapping as the attention kernel, so the slots are read as they were written.
+__global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, AttnSplit sp) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = lane >> 5, li = lane & 31;
+  const int nqb = (int)((p.sq[0] + p.sq[1] + QB - 1) / QB);
+  const int64_t Sq = p.sq[0] + p.sq[1];
+  const int nkb = (int)((p.skv[0] + p.skv[1] + KB - 1) / KB);
+  const int t = blockIdx.x;
+  const int first_piece = (t * nkb) / sp.len, last_piece = ((t + 1) * nkb - 1) / sp.len;
+  const int np = last_piece - first_piece + 1;
+  if (np == 1) return;  // the unit was covered by one piece, which wrote the output itself
+  const int unit = sp.full_units + t;
+  const int qblk = unit % nqb;
+  const int h = (unit / nqb) % p.heads, b = unit / (nqb * p.heads);
+  const float* base = sp.slots + (int64_t)t * sp.max_parts * kSlotFloats;
+  const int qi = wave * 32 + li;
+  float m = -INFINITY;
+  for (int i = 0; i < np; ++i) m = fmaxf(m, base[(int64_t)i * kSlotFloats + kSlotOFloats + QB + qi]);
+  f32x16 oacc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float l = 0.f;
+  for (int i = 0; i < np; ++i) {
+    const float* slot = base + (int64_t)i * kSlotFloats;
+    const float w = __builtin_amdgcn_exp2f(slot[kSlotOFloats + QB + qi] - m);
+    l += slot[kSlotOFloats + qi] * w;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(slot + ((((dt * 4 + rq) * 8 + wave) * 2 + g) * 32 + li) * 4);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) oacc[dt][4 * rq + c] += v[c] * w;
       }
   }
+  const int64_t row = (int64_t)qblk * QB + qi;
+  if (row < Sq) store_output(p, b, h, row, g, oacc, 1.0f / l);
 }
 
 }  // namespace
 
-int launch_attn_plain(const dsx_attn_params& p, hipStream_t st) {
+// Decides whether the last round of workgroups is worth splitting along the keys and lays the split out.
+// `cus` compute units, U units of nkb key blocks.  Returns the scratch bytes the split needs (0: no split).
+static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
+  const int64_t Sq = p.sq[0] + p.sq[1], Skv = p.skv[0] + p.skv[1];
+  const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
+  const int nkb = (int)((Skv + KB - 1) / KB);
+  sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr};
+  const int tail = (int)(units % cus);
+  const int64_t rounds = (units + cus - 1) / cus;
+  // Worth it when the compute units left idle in the last round are at least a quarter of the whole launch
+  // and the key axis is long enough for the parts to dwarf the cost of writing and merging them (~20 us).
+  // Below that the split loses: the chip is power-limited during attention, so a last round on fewer
+  // compute units runs at a higher clock (measured at 432 units on 256 compute units: 252 us whole,
+  // 265 us split; at 384 units: 218 us whole, 207 us split).
+  if (cus <= 0 || tail == 0 || nkb < 32 || (int64_t)(cus - tail) * 4 < rounds * cus) return 0;
+  sp.full_units = (int)(units - tail);
+  sp.tail_units = tail;
+  sp.pieces = cus;
+  sp.len = (int)(((int64_t)tail * nkb + cus - 1) / cus);
+  sp.max_parts = (nkb + sp.len - 1) / sp.len + 1;
+  return (int64_t)tail * sp.max_parts * kSlotFloats * (int64_t)sizeof(float);
+}
+
+static int device_cus() {
+  static int cus = -1;
+  if (cus < 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+    cus = prop.multiProcessorCount;
+  }
+  return cus;
+}
+
+int64_t attn_plain_workspace_bytes(const dsx_attn_params& p) {
+  AttnSplit sp;
+  return plan_split(p, device_cus(), sp);
+}
+
+// `scratch` / `scratch_bytes`: optional device memory for the key-range split (may be null).
+int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_bytes, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)attn_plain_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)attn_plain_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLdsBytes) != hipSuccess)
-      return DSX_ELAUNCH;
+    const void* kernels[4] = {(const void*)attn_plain_kernel<true, true>, (const void*)attn_plain_kernel<true, false>,
+                              (const void*)attn_plain_kernel<false, true>, (const void*)attn_plain_kernel<false, false>};
+    for (const void* kfn : kernels)
+      if (hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+        return DSX_ELAUNCH;
     attr_set = true;
   }
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
   if (units > (1ll << 30)) return DSX_EBADSHAPE;
-  dim3 grid((unsigned)(((units + 7) / 8) * 8)), block(512);
+  AttnSplit sp;
+  const int64_t need = plan_split(p, device_cus(), sp);
+  if (need == 0 || !scratch || scratch_bytes < need || ((uintptr_t)scratch & 15))
+    sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr};
+  else
+    sp.slots = (float*)scratch;
+  dim3 grid((unsigned)(((sp.full_units + 7) / 8) * 8 + sp.pieces)), block(512);
   // a caller-supplied bound on |softmax_scale * q.k| that keeps exp2 of every score inside fp32 and bf16
   // with a fixed reference lets the kernel skip the per-block maximum
   const bool bounded = p.score_bound > 0.f && p.score_bound * kLog2e <= kRescaleThreshold;
-  if (bounded)
-    attn_plain_kernel<false><<<grid, block, kLdsBytes, st>>>(p);
+  const bool split = sp.tail_units > 0;
+  if (bounded && split)
+    attn_plain_kernel<false, true><<<grid, block, kLdsBytes, st>>>(p, sp);
+  else if (bounded)
+    attn_plain_kernel<false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+  else if (split)
+    attn_plain_kernel<true, true><<<grid, block, kLdsBytes, st>>>(p, sp);
   else
-    attn_plain_kernel<true><<<grid, block, kLdsBytes, st>>>(p);
-  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+    attn_plain_kernel<true, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+  if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
+  if (sp.tail_units > 0) {
+    attn_merge_kernel<<<dim3((unsigned)sp.tail_units), block, 0, st>>>(p, sp);
+    if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
+  }
+  return DSX_OK;
 }
 
 }  // namespace dsx

@@ -250,11 +250,15 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
                 getattr(P, name)[i] = _ptr(w)
     P.norm_eps = eps
     P.score_bound = float(score_bound)
-    if keep and not in_kernel:
-        ws = torch.empty(2 * B * H * (S1 + S2 + Skv1 + Skv2) * D, dtype=torch.uint8, device=q.device)
-        keep.append(ws)
-        P.workspace, P.workspace_bytes = _ptr(ws), ws.numel()
-    rc = _lib.load().dsx_attn_fwd(P, _stream())
+    lib = _lib.load()
+    if not in_kernel:
+        # scratch for the one-off q/k pre-pass and for splitting the key range of a partly filled last round
+        need = lib.dsx_attn_workspace_bytes(P)
+        if need > 0:
+            ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+            keep.append(ws)
+            P.workspace, P.workspace_bytes = _ptr(ws), need
+    rc = lib.dsx_attn_fwd(P, _stream())
     _lib.check(rc, "dsx_attn_fwd")
     return (out, out2) if q2 is not None else out
 

@@ -176,15 +176,25 @@ typedef struct dsx_attn_params {
    * RMSNorm over head_dim with weights wq, wk: head_dim * max|wq| * max|wk| * softmax_scale.  A promise
    * that does not hold can overflow exp2. */
   float score_bound;
-  /* Optional scratch for the fused pre-processing, owned by the caller (NULL = none): when it holds at
-   * least 2*batch*heads*(Sq+Skv)*128 bytes, q and k are normalised/rotated ONCE into it by a row kernel
-   * and the attention kernel reads them from there; without it the same arithmetic is applied inside the
-   * attention kernel as tiles are loaded, where every query block repeats the work on K. */
+  /* Optional scratch owned by the caller (NULL = none, 16-byte aligned), used for two things when it is
+   * large enough (dsx_attn_workspace_bytes gives the size that enables both):
+   *  - fused pre-processing: with 2*batch*heads*(Sq+Skv)*128 bytes, q and k are normalised/rotated ONCE
+   *    into it by a row kernel and the attention kernel reads them from there; without it the same
+   *    arithmetic is applied inside the attention kernel as tiles are loaded, where every query block
+   *    repeats the work on K;
+   *  - load balance: when the (batch, head, 256-query block) units do not fill the last round of
+   *    workgroups, the key ranges of that round's units are cut into equal pieces over all compute units
+   *    and a second kernel merges the partial softmax results held in the scratch.
+   * Calls that share a scratch must not overlap. */
   void* workspace;
   int64_t workspace_bytes;
 } dsx_attn_params;
 
 int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
+
+/* Scratch bytes with which dsx_attn_fwd(p) uses every option described at `workspace` (0: none would be
+ * used).  Reads the shapes and the fused-option pointers of *p only; launches nothing. */
+int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p);
 
 /*
  * Standalone RMSNorm + RoPE of q and k (same arithmetic and rounding points as the fused

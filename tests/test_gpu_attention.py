@@ -206,3 +206,41 @@ def test_score_bound_promise_skips_the_running_maximum(dev, Sq, Skv):
     ignored = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=1e4).cpu()
     assert torch.equal(plain, bounded) and torch.equal(plain, ignored)
     assert _rel_err(bounded, want) <= TOL
+
+
+@pytest.mark.parametrize("H,Sq,Skv,qscale,bound", [(3, 2048, 2100, 1.0, 0.0), (2, 700, 4200, 12.0, 0.0),
+                                                   (5, 1000, 2048, 1.0, 0.0), (3, 2048, 2100, 0.25, 12.0)])
+def test_key_range_split_of_the_last_round(dev, H, Sq, Skv, qscale, bound):
+    """Few (head, query block) units and a long key axis: the launcher cuts the key ranges of the units into
+    equal pieces over all compute units and merges the partial softmax results.  Pieces end inside units and
+    span unit boundaries, the key axis is ragged, and with qscale > 1 the softmax references of the parts of
+    a row differ (scores beyond +-64 in the log2 domain), so the merge has to rescale."""
+    from diffsynth_engine_amd import _lib, ops
+
+    g = torch.Generator().manual_seed(H * Sq + Skv)
+    q = (torch.randn(1, H, Sq, 128, generator=g) * qscale).bfloat16()
+    k = torch.randn(1, H, Skv, 128, generator=g).bfloat16()
+    v = torch.randn(1, H, Skv, 128, generator=g).bfloat16()
+    want = O.sdpa(q.float(), k.float(), v.float())
+    P = _lib.AttnParams()
+    P.sq[0], P.skv[0], P.batch, P.heads, P.head_dim = Sq, Skv, 1, H, 128
+    assert _lib.load().dsx_attn_workspace_bytes(P) > 0  # this shape does take the split path
+    got = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=bound).cpu()
+    assert _rel_err(got, want) <= TOL
+    # the unsplit kernel (no scratch offered) gives the same rows up to the order of the fp32 sums
+    same = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=bound, in_kernel=True).cpu()
+    assert _rel_err(got, same) <= 2 ** -7
+
+
+def test_key_range_split_joint_two_segments(dev):
+    """The split also has to honour the two-segment (text + image) addressing of q, k, v and o."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(5)
+    H, S1, S2 = 4, 512, 1792
+    mk = lambda s: torch.randn(1, H, s, 128, generator=g).bfloat16()
+    q1, k1, v1, q2, k2, v2 = mk(S1), mk(S1), mk(S1), mk(S2), mk(S2), mk(S2)
+    want = O.sdpa(torch.cat([q1, q2], 2).float(), torch.cat([k1, k2], 2).float(), torch.cat([v1, v2], 2).float())
+    o1, o2 = ops.attention_bhsd(q1.to(dev), k1.to(dev), v1.to(dev), q2=q2.to(dev), k2=k2.to(dev), v2=v2.to(dev))
+    got = torch.cat([o1, o2], 2).cpu()
+    assert _rel_err(got, want) <= TOL
