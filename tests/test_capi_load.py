@@ -120,3 +120,13 @@ def test_fp8_inference_patches_and_restores_f_linear():
         with fp8_inference(True):
             raise KeyError("boom")
     assert F.linear is orig
+
+
+def test_graft_entry_build_checks_pass_on_the_built_library(monkeypatch):
+    """build() compiles and then checks the import and the ABI version; here the compile step is skipped and
+    the checks run against the library already in the tree."""
+    import __graft_entry__ as entry
+    from diffsynth_engine_amd import build as build_mod
+
+    monkeypatch.setattr(build_mod, "build_library", lambda verbose=True: build_mod.LIB_PATH)
+    entry.build()
