@@ -1,0 +1,115 @@
+"""GPU checks at the benchmark's full sizes (4608 tokens, 24 heads, the four GEMM shapes of the FP8 linear
+micro-benchmark), through properties that do not need a CPU pass over the whole problem: independence of
+rows, exact scaling by powers of two, exactness on small integers, softmax invariants, and agreement with
+torch's own fp32 routines evaluated on the device for a slice."""
+import math
+
+import pytest
+import torch
+
+from oracle import dit_ops as O
+from oracle import fp8 as ofp8
+
+pytestmark = pytest.mark.gpu
+
+M_FULL = 4608
+GEMM_SHAPES = [(3072, 9216), (3072, 3072), (3072, 12288), (12288, 3072)]  # (K, N) at M = 4608
+
+
+def _operands(dev, K, N, seed):
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    x = torch.randn(M_FULL, K, generator=g, device=dev, dtype=torch.bfloat16)
+    x[:, torch.randperm(K, generator=g, device=dev)[: max(1, -(-K // 1000))]] *= 20  # a few outlier channels
+    w = (torch.randn(N, K, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    bias = torch.randn(N, generator=g, device=dev).to(torch.bfloat16)
+    wq, ws = ops.quantize_weight_fp8(w)
+    xq, xs = ops.quantize_fp8(x)
+    return x, xq, xs, wq, ws, bias
+
+
+@pytest.mark.parametrize("K,N", GEMM_SHAPES)
+def test_full_size_gemm_against_dequantised_matmul(dev, K, N):
+    """cosine >= 0.9995 against the fp32 product of the dequantised operands (torch on the device), and the
+    quantiser's codes and scales equal to the oracle's on a slice of rows."""
+    from diffsynth_engine_amd import ops
+
+    x, xq, xs, wq, ws, bias = _operands(dev, K, N, seed=K + N)
+    got = ops.fp8_gemm(xq, wq, xs, ws, bias)
+    ref = (xq.float() * xs[:, None]) @ (wq.float() * ws).t() + bias.float()
+    cos = torch.nn.functional.cosine_similarity(got.float().flatten(), ref.flatten(), dim=0).item()
+    assert cos >= 0.9995, cos
+    # every element within bf16 rounding of the fp32 reference (fp32 accumulation order differs)
+    tol = ref.abs() * 2 ** -7 + 2 ** -6
+    assert bool(((got.float() - ref).abs() <= tol).all())
+    rows = slice(1000, 1064)
+    oq, osc = ofp8.quantize_rowwise(x[rows].cpu(), scaled=True)
+    assert torch.equal(xq[rows].cpu().view(torch.uint8), oq.view(torch.uint8)) and torch.equal(xs[rows].cpu(), osc)
+
+
+def test_full_size_gemm_rows_are_independent_and_scales_are_linear(dev):
+    """Rows 1024..1279 of the full problem equal the same rows computed as a 256-row problem, bit for bit (same
+    tile, same accumulation order); doubling every activation scale doubles the bias-free output exactly."""
+    from diffsynth_engine_amd import ops
+
+    K, N = 3072, 9216
+    _, xq, xs, wq, ws, bias = _operands(dev, K, N, seed=3)
+    full = ops.fp8_gemm(xq, wq, xs, ws, bias)
+    part = ops.fp8_gemm(xq[1024:1280], wq, xs[1024:1280], ws, bias)
+    assert torch.equal(full[1024:1280], part)
+    plain = ops.fp8_gemm(xq, wq, xs, ws, None)
+    doubled = ops.fp8_gemm(xq, wq, xs * 2, ws, None)
+    assert torch.equal(doubled.float(), plain.float() * 2)
+
+
+def test_full_size_gemm_exact_on_small_integers(dev):
+    """Operands that are small integers in e4m3 and unit scales: every product and partial sum is an integer
+    below 2^24, so the result is exact whatever the order of accumulation."""
+    from diffsynth_engine_amd import ops
+
+    K, N = 3072, 3072
+    g = torch.Generator(device=dev).manual_seed(5)
+    a = torch.randint(-3, 4, (M_FULL, K), generator=g, device=dev).to(torch.float32)
+    w = torch.randint(-2, 3, (N, K), generator=g, device=dev).to(torch.float32)
+    aq, wq = a.to(torch.float8_e4m3fn), w.to(torch.float8_e4m3fn)
+    got = ops.fp8_gemm(aq, wq, None, None, None)
+    want = (a @ w.t()).to(torch.bfloat16)  # |sum| <= 18432 < 2^24: the fp32 matmul is exact too
+    assert torch.equal(got, want)
+
+
+def test_full_size_attention_invariants(dev):
+    """S = 4608, 24 heads.  (1) constant V gives that constant back; (2) permuting the keys (and values with
+    them) changes nothing beyond the order of the fp32 sums; (3) two heads agree with torch's fp32 SDPA on the
+    device."""
+    from diffsynth_engine_amd import ops
+
+    H, S = 24, 4608
+    g = torch.Generator(device=dev).manual_seed(9)
+    q, k, v = [torch.randn(1, H, S, 128, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(3)]
+    ones = torch.full_like(v, 0.75)
+    out = ops.attention_bhsd(q, k, ones)
+    assert bool(((out.float() - 0.75).abs() <= 0.75 * 2 ** -7).all())  # sum of bf16 P over fp32 sum of P
+    base = ops.attention_bhsd(q, k, v)
+    perm = torch.randperm(S, generator=g, device=dev)
+    shuffled = ops.attention_bhsd(q, k[:, :, perm], v[:, :, perm])
+    scale = base.float().abs().max()
+    assert ((shuffled.float() - base.float()).abs().max() / scale).item() <= 2 ** -6
+    ref = torch.nn.functional.scaled_dot_product_attention(q[:, 5:7].float(), k[:, 5:7].float(), v[:, 5:7].float())
+    err = ((base[:, 5:7].float() - ref).abs().max() / ref.abs().max()).item()
+    assert err <= 2e-2, err
+
+
+def test_full_size_attention_first_rows_match_cpu_oracle(dev):
+    """A handful of query rows of one head at S = 4608 against the CPU oracle (the rest of the row space is
+    covered by the invariants above)."""
+    from diffsynth_engine_amd import ops
+
+    S = 4608
+    g = torch.Generator().manual_seed(10)
+    q, k, v = [torch.randn(1, 1, S, 128, generator=g).bfloat16() for _ in range(3)]
+    got = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev)).cpu()
+    rows = torch.tensor([0, 1, 255, 256, 2303, 4607])
+    want = O.sdpa(q[:, :, rows].float(), k.float(), v.float())
+    err = ((got[:, :, rows].float() - want).abs().max() / want.abs().max()).item()
+    assert err <= 2e-2, err
