@@ -11,7 +11,8 @@ flops): algorithmic flops 2*M*N*K of every large GEMM launched in the timed regi
 their durations, measured with events on the launch stream.  `cpu_baseline` times the CPU oracle
 (pure-torch restatement of the reference path) on the host cores for a bounded sample.
 Secondary figures (attention kernel TFLOP/s at S=4608, per-shape GEMM TFLOP/s, HBM GB/s of the
-bandwidth-bound kernels) ride along under "detail".
+bandwidth-bound kernels) ride along under "detail".  `--workload wan14b` times one Wan2.1-14B step instead
+(40 layers, 32 760 video tokens) and prints its own line.
 """
 import argparse
 import json
@@ -76,6 +77,80 @@ def flux_state_dict_stream(num_double, num_single, device, seed=0, std=0.02):
         yield from lin(p + "proj_out", 5 * d, d)
     yield from lin("final_norm_out.linear", d, 2 * d)
     yield from lin("final_proj_out", d, 64)
+
+
+def wan_state_dict_stream(cfg, device, seed=0, std=0.02):
+    """(name, tensor) pairs of a random Wan2.1-architecture DiT (text-to-video variant), generated on the
+    device one tensor at a time: Linear weights N(0,std) bf16, biases 0, norm weights 1, modulation tables
+    N(0,1)/sqrt(dim)."""
+    import torch
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    d, f = cfg["dim"], cfg["ffn_dim"]
+    bf = torch.bfloat16
+
+    def lin(name, n_in, n_out):
+        yield name + ".weight", (torch.randn(n_out, n_in, generator=g, device=device) * std).to(bf)
+        yield name + ".bias", torch.zeros(n_out, dtype=bf, device=device)
+
+    pf, ph, pw = cfg["patch_size"]
+    yield "patch_embedding.weight", (torch.randn(d, cfg["in_dim"], pf, ph, pw, generator=g, device=device) * std).to(bf)
+    yield "patch_embedding.bias", torch.zeros(d, dtype=bf, device=device)
+    yield from lin("text_embedding.0", cfg["text_dim"], d)
+    yield from lin("text_embedding.2", d, d)
+    yield from lin("time_embedding.0", cfg["freq_dim"], d)
+    yield from lin("time_embedding.2", d, d)
+    yield from lin("time_projection.1", d, 6 * d)
+    for i in range(cfg["num_layers"]):
+        p = f"blocks.{i}."
+        for a in ("self_attn", "cross_attn"):
+            for n in ("q", "k", "v", "o"):
+                yield from lin(p + f"{a}.{n}", d, d)
+            yield p + f"{a}.norm_q.weight", torch.ones(d, dtype=bf, device=device)
+            yield p + f"{a}.norm_k.weight", torch.ones(d, dtype=bf, device=device)
+        yield p + "norm3.weight", torch.ones(d, dtype=bf, device=device)
+        yield p + "norm3.bias", torch.zeros(d, dtype=bf, device=device)
+        yield from lin(p + "ffn.0", d, f)
+        yield from lin(p + "ffn.2", f, d)
+        yield p + "modulation", (torch.randn(1, 6, d, generator=g, device=device) / d ** 0.5).to(bf)
+    yield from lin("head.head", d, cfg["out_dim"] * pf * ph * pw)
+    yield "head.modulation", (torch.randn(1, 2, d, generator=g, device=device) / d ** 0.5).to(bf)
+
+
+def run_wan(args, torch, dev):
+    """BASELINE configs[4]: one Wan2.1-14B DiT denoising step, 21 x 60 x 104 latent = 32 760 tokens, 512 text
+    tokens, 40 layers; every Linear through the scaled e4m3 GEMM."""
+    from diffsynth_engine_amd.wan_dit import WanDiTRunner
+
+    cfg = dict(dim=5120, in_dim=16, ffn_dim=13824, out_dim=16, text_dim=4096, freq_dim=256, eps=1e-6,
+               patch_size=(1, 2, 2), num_heads=40, num_layers=args.wan_layers)
+    runner = WanDiTRunner(wan_state_dict_stream(cfg, dev), cfg, scaled=True, device=dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(1, 16, 21, 60, 104, generator=g, device=dev).to(torch.bfloat16)
+    ctx = torch.randn(1, 512, 4096, generator=g, device=dev).to(torch.bfloat16)
+    t = torch.tensor([500.0], device=dev)
+    for _ in range(args.warmup):
+        out = runner(x, ctx, t)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = runner(x, ctx, t)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert torch.isfinite(out.float()).all().item(), "non-finite output"
+    S, d, f, L = 21 * 30 * 52, cfg["dim"], cfg["ffn_dim"], cfg["num_layers"]
+    gemm = L * (2.0 * S * d * d * 4 + 2.0 * S * d * f * 2 + 2.0 * S * d * d * 2 + 2.0 * 512 * d * d * 2)
+    attn = L * (4.0 * S * S * d + 4.0 * S * 512 * d)
+    t_ideal = gemm / PEAK_FP8 + attn / PEAK_BF16
+    print(json.dumps({
+        "metric": "wan2.1_14b_480p_fp8_dit_step_ms", "value": round(ms, 1), "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 1), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 GEMM (fp32 accumulate) + bf16 attention",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE configs[4]: Wan2.1-14B-architecture DiT, one denoising step, %d layers, "
+                               "32760 video tokens (21x60x104 latent) + 512 text tokens, batch 1, random init" % L},
+        "step_roofline": {"algorithmic_tflop": round((gemm + attn) / 1e12, 1), "ideal_ms": round(t_ideal * 1e3, 1),
+                          "frac": round(t_ideal * 1e3 / ms, 4)}}))
 
 
 def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
@@ -273,6 +348,9 @@ def main():
     ap.add_argument("--single", type=int, default=38)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
+    ap.add_argument("--workload", choices=("flux", "wan14b"), default="flux",
+                    help="flux (default): the headline Flux-1024 step; wan14b: one Wan2.1-14B step (configs[4])")
+    ap.add_argument("--wan-layers", type=int, default=40)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size dispatch that FETCH_SIZE / "
                          "WRITE_SIZE counter runs are scaled by")
@@ -292,6 +370,8 @@ def main():
         sys.exit("bench.py: " + _lib.strerror(rc))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "wan14b":
+        return run_wan(args, torch, dev)
 
     runner = FluxDiTRunner(flux_state_dict_stream(args.double, args.single, dev), args.double, args.single,
                            scaled=True, device=dev)
