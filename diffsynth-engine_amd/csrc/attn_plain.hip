@@ -89,7 +89,10 @@ __device__ __forceinline__ void store_output(const dsx_attn_params& p, int b, in
 // reference can stay 0 for the whole row and the per-block maximum is not computed at all.
 // SPLIT = false: every workgroup runs one whole unit (sp.full_units = all of them); the loop over parts
 // and the variable key range fold away.
-template <bool SCAN, bool SPLIT>
+// QPRE = true: q still needs its RMSNorm (p.q_norm_w) and / or RoPE (p.rope); they are applied to the
+// workgroup's 256 query rows as they are loaded, which is free (each q row is read exactly once).  K is
+// read by every query block of its head, so the same work on k belongs in a one-off pass before this kernel.
+template <bool SCAN, bool SPLIT, bool QPRE>
 __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, AttnSplit sp) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x;
@@ -231,9 +234,27 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
     if (row >= Sq) row = Sq - 1;
     const int seg = row >= p.sq[0] ? 1 : 0;
     const uint16_t* src = qbase[seg] + (row - (seg ? p.sq[0] : 0)) * p.q_ss[seg];
+    u32x4 raws[8];
+#pragma unroll
+    for (int kc = 0; kc < 8; ++kc) raws[kc] = *reinterpret_cast<const u32x4*>(src + kc * 16 + g * 8);
+    if (QPRE) {
+      const uint16_t* nw = (const uint16_t*)p.q_norm_w[seg];
+      const float* rope = p.rope ? p.rope + (int64_t)b * p.rope_sb + row * HD : nullptr;
+      float rrms = 1.f;
+      if (nw) {
+        float ss = 0.f;
+#pragma unroll
+        for (int kc = 0; kc < 8; ++kc) ss += sumsq_chunk(raws[kc]);
+        rrms = rsqrtf(pair_sum(ss) * (1.0f / HD) + p.norm_eps);
+      }
+#pragma unroll
+      for (int kc = 0; kc < 8; ++kc)
+        raws[kc] = norm_rope_chunk(raws[kc], nw != nullptr, rrms, nw ? nw + kc * 16 + g * 8 : nullptr,
+                                   rope ? rope + kc * 16 + g * 8 : nullptr);
+    }
 #pragma unroll
     for (int kc = 0; kc < 8; ++kc) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(src + kc * 16 + g * 8);
+      const u32x4 raw = raws[kc];
       u32x4 sc;
       sc.x = pack_bf16x2(bf16_lo(raw.x) * c, bf16_hi(raw.x) * c);
       sc.y = pack_bf16x2(bf16_lo(raw.y) * c, bf16_hi(raw.y) * c);
@@ -557,6 +578,7 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
   const int nkb = (int)((Skv + KB - 1) / KB);
   sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr};
+  if (p.rope || p.q_norm_w[0] || p.q_norm_w[1]) return 0;  // the split kernel has no q pre-processing
   const int tail = (int)(units % cus);
   const int64_t rounds = (units + cus - 1) / cus;
   // Worth it when the compute units left idle in the last round are at least a quarter of the whole launch
@@ -593,8 +615,10 @@ int64_t attn_plain_workspace_bytes(const dsx_attn_params& p) {
 int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_bytes, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    const void* kernels[4] = {(const void*)attn_plain_kernel<true, true>, (const void*)attn_plain_kernel<true, false>,
-                              (const void*)attn_plain_kernel<false, true>, (const void*)attn_plain_kernel<false, false>};
+    const void* kernels[6] = {
+        (const void*)attn_plain_kernel<true, true, false>,   (const void*)attn_plain_kernel<false, true, false>,
+        (const void*)attn_plain_kernel<true, false, false>,  (const void*)attn_plain_kernel<false, false, false>,
+        (const void*)attn_plain_kernel<true, false, true>,   (const void*)attn_plain_kernel<false, false, true>};
     for (const void* kfn : kernels)
       if (hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
         return DSX_ELAUNCH;
@@ -614,14 +638,19 @@ int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_b
   // with a fixed reference lets the kernel skip the per-block maximum
   const bool bounded = p.score_bound > 0.f && p.score_bound * kLog2e <= kRescaleThreshold;
   const bool split = sp.tail_units > 0;
-  if (bounded && split)
-    attn_plain_kernel<false, true><<<grid, block, kLdsBytes, st>>>(p, sp);
+  const bool qpre = p.rope || p.q_norm_w[0] || p.q_norm_w[1];  // (never together with the split)
+  if (qpre && bounded)
+    attn_plain_kernel<false, false, true><<<grid, block, kLdsBytes, st>>>(p, sp);
+  else if (qpre)
+    attn_plain_kernel<true, false, true><<<grid, block, kLdsBytes, st>>>(p, sp);
+  else if (bounded && split)
+    attn_plain_kernel<false, true, false><<<grid, block, kLdsBytes, st>>>(p, sp);
   else if (bounded)
-    attn_plain_kernel<false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+    attn_plain_kernel<false, false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
   else if (split)
-    attn_plain_kernel<true, true><<<grid, block, kLdsBytes, st>>>(p, sp);
+    attn_plain_kernel<true, true, false><<<grid, block, kLdsBytes, st>>>(p, sp);
   else
-    attn_plain_kernel<true, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+    attn_plain_kernel<true, false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
   if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
   if (sp.tail_units > 0) {
     attn_merge_kernel<<<dim3((unsigned)sp.tail_units), block, 0, st>>>(p, sp);

@@ -100,7 +100,9 @@ class FluxDiTRunner:
                  device="cuda:0", fuse_rope_in_attention: bool = False):
         self.device = torch.device(device)
         self.scaled = scaled
-        # True: RMSNorm/RoPE applied inside the attention kernel's tile loads; False: one in-place pre-pass
+        # q/k RMSNorm and RoPE are requested from the attention entry point.  False (default): the library
+        # gets scratch, treats k once in a row pass and q as the attention kernel loads it; True: no scratch,
+        # everything inside the attention kernel's tile loads (every query block repeats the work on k)
         self.fuse_rope_in_attention = fuse_rope_in_attention
         self.num_double, self.num_single = num_double, num_single
         self.lin: Dict[str, _Linear] = {}
@@ -216,27 +218,18 @@ class FluxDiTRunner:
         qkv_a, qkv_b = _gemm_pair(L[pre + "attn.a_to_qkv"], dict(a_q=qa.view(-1, d), a_s=sa),
                                   L[pre + "attn.b_to_qkv"], dict(a_q=qb.view(-1, d), a_s=sb))
         nw = self.norm_w
-        if not self.fuse_rope_in_attention:
-            # RMSNorm + RoPE rewrite q and k in place inside the packed projections (one read + one write of
-            # q and k) so that the attention kernel streams K without re-normalising it once per query tile
-            ops.rmsnorm_rope_qk(qkv_b.view(B, St, 3 * d), HEADS, HEADS, nw[pre + "attn.norm_q_b"],
-                                nw[pre + "attn.norm_k_b"], rope, 0, EPS)
-            ops.rmsnorm_rope_qk(qkv_a.view(B, Si, 3 * d), HEADS, HEADS, nw[pre + "attn.norm_q_a"],
-                                nw[pre + "attn.norm_k_a"], rope, St, EPS)
         qkv_a = qkv_a.view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         qkv_b = qkv_b.view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         qb_, kb_, vb_ = qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:]
         qa_, ka_, va_ = qkv_a[:, :HEADS], qkv_a[:, HEADS:2 * HEADS], qkv_a[:, 2 * HEADS:]
-        if self.fuse_rope_in_attention:
-            ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, rope=rope,
-                               q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
-                               q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
-                               out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2), in_kernel=True)
-        else:
-            ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2),
-                               out2=o_a.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
+        # joint attention over [text; image] rows with the per-stream q/k RMSNorm weights and the RoPE table
+        ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, rope=rope,
+                           q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
+                           q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
+                           out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2),
+                           in_kernel=self.fuse_rope_in_attention, score_bound=self.score_bound.get(pre, 0.0))
         # The two streams run the same sequence on different weights (flux_dit.py:226-234): out-projection +
         # gated residual, LN-modulate, MLP + gated residual.  Each pair of linears goes out as one grouped
         # submission so that the 512-token text problem runs beside the image problem instead of after it.
@@ -267,13 +260,9 @@ class FluxDiTRunner:
         qkv = h.view(B, S, 7 * d)[:, :, : 3 * d].unflatten(2, (3 * HEADS, HEAD_DIM)).transpose(1, 2)
         nw = self.norm_w
         q_, k_, v_ = qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:]
-        if self.fuse_rope_in_attention:
-            ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
-                               eps=EPS, out=att.transpose(1, 2), in_kernel=True)
-        else:
-            ops.rmsnorm_rope_qk(h.view(B, S, 7 * d), HEADS, HEADS, nw[pre + "norm_q_a"], nw[pre + "norm_k_a"], rope,
-                                0, EPS)
-            ops.attention_bhsd(q_, k_, v_, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
+        ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
+                           eps=EPS, out=att.transpose(1, 2), in_kernel=self.fuse_rope_in_attention,
+                           score_bound=self.score_bound.get(pre, 0.0))
         # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
         # parts and emits the e4m3 operand of proj_out with its per-token scale
         if self.scaled:

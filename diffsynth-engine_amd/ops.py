@@ -202,7 +202,7 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     in_kernel: offer the library no scratch buffer.  RoPE / RMSNorm are then applied inside the attention kernel
     as tiles are loaded (every query block repeats the work on K) and the key range of a sparsely filled last
     round of workgroups is not split.  Default: a scratch buffer of dsx_attn_workspace_bytes is allocated here;
-    q and k are normalised / rotated once into it.
+    k is normalised / rotated once into it and q as the attention kernel loads it.
     score_bound: optional promise |scale * q.k| <= score_bound for every pair (after RMSNorm/RoPE); when it is
     small enough the kernel skips the running softmax maximum (same result).  0 = no promise.
     Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).

@@ -178,10 +178,10 @@ typedef struct dsx_attn_params {
   float score_bound;
   /* Optional scratch owned by the caller (NULL = none, 16-byte aligned), used for two things when it is
    * large enough (dsx_attn_workspace_bytes gives the size that enables both):
-   *  - fused pre-processing: with 2*batch*heads*(Sq+Skv)*128 bytes, q and k are normalised/rotated ONCE
-   *    into it by a row kernel and the attention kernel reads them from there; without it the same
-   *    arithmetic is applied inside the attention kernel as tiles are loaded, where every query block
-   *    repeats the work on K;
+   *  - fused pre-processing: with 2*batch*heads*Skv*128 bytes, k is normalised/rotated ONCE into it by a
+   *    row kernel and the attention kernel reads it from there (q is treated as it is loaded, each row
+   *    once); without it the same arithmetic is applied inside the attention kernel as tiles are loaded,
+   *    where every query block repeats the work on K;
    *  - load balance: when the (batch, head, 256-query block) units do not fill the last round of
    *    workgroups, the key ranges of that round's units are cut into equal pieces over all compute units
    *    and a second kernel merges the partial softmax results held in the scratch.
