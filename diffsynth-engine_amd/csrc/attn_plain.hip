@@ -579,6 +579,7 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   const int nkb = (int)((Skv + KB - 1) / KB);
   sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr};
   if (p.rope || p.q_norm_w[0] || p.q_norm_w[1]) return 0;  // the split kernel has no q pre-processing
+  if (cus <= 0) return 0;                                    // no device to ask
   const int tail = (int)(units % cus);
   const int64_t rounds = (units + cus - 1) / cus;
   // Worth it when the compute units left idle in the last round are at least a quarter of the whole launch
@@ -586,7 +587,7 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   // Below that the split loses: the chip is power-limited during attention, so a last round on fewer
   // compute units runs at a higher clock (measured at 432 units on 256 compute units: 252 us whole,
   // 265 us split; at 384 units: 218 us whole, 207 us split).
-  if (cus <= 0 || tail == 0 || nkb < 32 || (int64_t)(cus - tail) * 4 < rounds * cus) return 0;
+  if (tail == 0 || nkb < 32 || (int64_t)(cus - tail) * 4 < rounds * cus) return 0;
   sp.full_units = (int)(units - tail);
   sp.tail_units = tail;
   sp.pieces = cus;

@@ -130,3 +130,25 @@ def test_graft_entry_build_checks_pass_on_the_built_library(monkeypatch):
 
     monkeypatch.setattr(build_mod, "build_library", lambda verbose=True: build_mod.LIB_PATH)
     entry.build()
+
+
+def test_attention_workspace_size_query():
+    """dsx_attn_workspace_bytes needs no GPU: with RoPE / q-k RMSNorm requested it asks for the bf16 copy of k
+    (q is treated inside the attention kernel), otherwise (no GPU to split work over) for nothing."""
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    P = _lib.AttnParams()
+    P.sq[0], P.sq[1], P.skv[0], P.skv[1] = 512, 4096, 512, 4096
+    P.batch, P.heads, P.head_dim = 2, 24, 128
+    if not torch.cuda.is_available():
+        assert lib.dsx_attn_workspace_bytes(P) == 0
+    buf = ctypes.create_string_buffer(64)
+    P.k_norm_w[0] = ctypes.addressof(buf)
+    need = lib.dsx_attn_workspace_bytes(P)
+    assert need >= 2 * 2 * 24 * 4608 * 128
+    if not torch.cuda.is_available():
+        assert need == 2 * 2 * 24 * 4608 * 128
+    P.head_dim = 64
+    assert lib.dsx_attn_workspace_bytes(P) == 0
+    assert lib.dsx_attn_workspace_bytes(None) == 0
