@@ -332,9 +332,10 @@ extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale,
       (const uint16_t*)x, ldx, (const uint16_t*)scale, (const uint16_t*)shift, mod_sb,             \
       rows_per_batch, (const uint16_t*)ln_w, (const uint16_t*)ln_b, eps, (uint16_t*)y, ldy,        \
       (uint8_t*)q, ldq, q_scale, rows, (int)D)
-  // one wavefront per row while a row fits 12 chunks per lane and there are rows enough to fill the chip
+  // One wavefront per row while a row fits 6 chunks per lane and there are rows enough to fill the chip.
+  // Wider rows go to a workgroup per row: 12 chunks per lane cost 217 registers, two waves per SIMD and
+  // 266 us for 32760 x 5120; the workgroup form takes 160 us.
   if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_ADALN(6, 64);
-  else if (D <= 512 * 12 && rows >= 1024) DSX_LAUNCH_ADALN(12, 64);
   else if (D <= 2048 * 2) DSX_LAUNCH_ADALN(2, 256);
   else if (D <= 2048 * 3) DSX_LAUNCH_ADALN(3, 256);
   else DSX_LAUNCH_ADALN(8, 256);
@@ -446,7 +447,7 @@ extern "C" int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float
       (const uint16_t*)x, ldx, (const uint16_t*)w, eps, rope, rope_sb, rows_per_batch, (uint16_t*)out, ldo,   \
       rows, (int)D)
   if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_RMS(6, 64);
-  else if (D <= 512 * 12 && rows >= 1024) DSX_LAUNCH_RMS(12, 64);
+  else if (D <= 2048 * 3) DSX_LAUNCH_RMS(3, 256);
   else DSX_LAUNCH_RMS(8, 256);
 #undef DSX_LAUNCH_RMS
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
