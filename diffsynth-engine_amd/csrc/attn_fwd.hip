@@ -429,6 +429,8 @@ extern "C" int dsx_attn_fwd(const dsx_attn_params* p, void* stream) {
   // With caller scratch: k is normalised / rotated ONCE into it by a row kernel (every query block of a
   // head reads all of k), while q gets the same treatment for free inside the attention kernel, where each
   // row is read exactly once.
+  const bool k_side = p->rope || p->k_norm_w[0] || p->k_norm_w[1];
+  if (!k_side) return launch_attn_plain(*p, nullptr, 0, (hipStream_t)stream);  // q only: nothing to copy
   const int64_t ws_need = 2 * (int64_t)p->batch * p->heads * Skv * HD;
   if (p->workspace && p->workspace_bytes >= ws_need) {
     hipStream_t st = (hipStream_t)stream;
@@ -525,7 +527,7 @@ extern "C" int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p) {
   if (!p || p->head_dim != HD || p->batch <= 0 || p->heads <= 0) return 0;
   const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
   if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 30) || Skv > (1ll << 30)) return 0;
-  const bool fused = p->rope || p->q_norm_w[0] || p->q_norm_w[1] || p->k_norm_w[0] || p->k_norm_w[1];
-  const int64_t copies = fused ? 2 * (int64_t)p->batch * p->heads * Skv * HD : 0;
+  const bool k_side = p->rope || p->k_norm_w[0] || p->k_norm_w[1];
+  const int64_t copies = k_side ? 2 * (int64_t)p->batch * p->heads * Skv * HD : 0;
   return copies + attn_plain_workspace_bytes(*p);
 }

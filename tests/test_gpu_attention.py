@@ -244,3 +244,22 @@ def test_key_range_split_joint_two_segments(dev):
     o1, o2 = ops.attention_bhsd(q1.to(dev), k1.to(dev), v1.to(dev), q2=q2.to(dev), k2=k2.to(dev), v2=v2.to(dev))
     got = torch.cat([o1, o2], 2).cpu()
     assert _rel_err(got, want) <= TOL
+
+
+def test_q_only_rmsnorm_needs_no_scratch(dev):
+    """RMSNorm requested for q alone: the attention kernel applies it as it loads the query rows, no copy of k
+    is made and no scratch is asked for."""
+    from diffsynth_engine_amd import _lib, ops
+
+    g = torch.Generator().manual_seed(21)
+    q, k, v = [torch.randn(1, 2, 200, 128, generator=g).bfloat16() for _ in range(3)]
+    w = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16()
+    qn = O.rms_norm(q, w, 1e-6)
+    want = O.sdpa(qn.float(), k.float(), v.float())
+    P = _lib.AttnParams()
+    P.sq[0], P.skv[0], P.batch, P.heads, P.head_dim = 200, 200, 1, 2, 128
+    wd = w.to(dev)
+    P.q_norm_w[0] = wd.data_ptr()
+    assert _lib.load().dsx_attn_workspace_bytes(P) == 0
+    got = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), q_norm_w=wd).cpu()
+    assert _rel_err(got, want) <= TOL
