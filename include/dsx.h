@@ -193,7 +193,8 @@ typedef struct dsx_attn_params {
 int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
 
 /* Scratch bytes with which dsx_attn_fwd(p) uses every option described at `workspace` (0: none would be
- * used).  Reads the shapes and the fused-option pointers of *p only; launches nothing. */
+ * used).  Reads the shapes and the fused-option pointers of *p only; launches nothing.  No counterpart in
+ * the reference, whose attention backends allocate their own temporaries. */
 int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p);
 
 /*
