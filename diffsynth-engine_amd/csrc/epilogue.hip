@@ -63,14 +63,11 @@ __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint1
     }
   }
   if (q) {
-    float amax = 0.f;
+    float amax = 0.f;  // slots past the end of the row hold zeros (callers see to that)
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = t + i * TPR;
-      if (c < nchunk) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(val[i][j]));
-      }
+      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(val[i][j]));
     }
     amax = fmaxf(row_max<TPR>(amax, red), 1e-12f);
     const float inv = 448.0f / amax;
@@ -96,72 +93,108 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
   const bool live = row < rows;  // only possible to fail for TPR == 64 (whole wavefront idle)
   if (!live) row = rows - 1;
   const int nchunk = D >> 3;
+  // Chunk slots past the end of the row are clamped onto its last chunk, so that no load sits under a
+  // lane predicate: the compiler then issues a row's loads back to back instead of waiting for each.
+  int cc[NCH];
+  bool ok[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = t + i * TPR;
+    ok[i] = c < nchunk;
+    cc[i] = min(c, nchunk - 1);
+  }
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  const int64_t bidx = row / rows_per_batch;
+  const u32x4* sc = scale ? reinterpret_cast<const u32x4*>(scale + bidx * mod_sb) : nullptr;
+  const u32x4* sh = shift ? reinterpret_cast<const u32x4*>(shift + bidx * mod_sb) : nullptr;
+  u32x4 raw[NCH], sraw[NCH], hraw[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) raw[i] = xr[cc[i]];
+  // the modulation vectors are L2 hits (every row of a batch entry reads the same ones); fetched here, they
+  // arrive under the two row reductions
+  if (sc) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) sraw[i] = sc[cc[i]];
+  }
+  if (sh) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) hraw[i] = sh[cc[i]];
+  }
   float val[NCH][8];
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = t + i * TPR;
-    if (c < nchunk) {
-      u32x4 w = xr[c];
-      unpack8(w, val[i]);
+    unpack8(raw[i], val[i]);
+    float part = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) sum += val[i][j];
-    }
+    for (int j = 0; j < 8; ++j) part += val[i][j];
+    sum += ok[i] ? part : 0.f;
   }
   const float mean = row_sum<TPR>(sum, red) / (float)D;
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = t + i * TPR;
-    if (c < nchunk) {
+    float part = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float d = val[i][j] - mean;
-        sq += d * d;
-      }
+    for (int j = 0; j < 8; ++j) {
+      const float d = val[i][j] - mean;
+      part += d * d;
     }
+    sq += ok[i] ? part : 0.f;
   }
   const float rstd = rsqrtf(row_sum<TPR>(sq, red) / (float)D + eps);
-  const int64_t bidx = row / rows_per_batch;
-  const u32x4* sc = scale ? reinterpret_cast<const u32x4*>(scale + bidx * mod_sb) : nullptr;
-  const u32x4* sh = shift ? reinterpret_cast<const u32x4*>(shift + bidx * mod_sb) : nullptr;
+  const bool ragged = nchunk != NCH * TPR;  // uniform
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = t + i * TPR;
-    if (c < nchunk) {
-      float v[8];
+    float v[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = (val[i][j] - mean) * rstd;
-      if (ln_w) {
-        float w[8];
-        unpack8(reinterpret_cast<const u32x4*>(ln_w)[c], w);
+    for (int j = 0; j < 8; ++j) v[j] = (val[i][j] - mean) * rstd;
+    if (ln_w) {
+      float w[8];
+      unpack8(reinterpret_cast<const u32x4*>(ln_w)[cc[i]], w);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] *= w[j];
-      }
-      if (ln_b) {
-        float bb[8];
-        unpack8(reinterpret_cast<const u32x4*>(ln_b)[c], bb);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] += bb[j];
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j]);  // LayerNorm output tensor (bf16)
-      if (sc) {
-        float s8[8];
-        unpack8(sc[c], s8);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j] * round_bf16(1.0f + s8[j]));
-      }
-      if (sh) {
-        float h8[8];
-        unpack8(sh[c], h8);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = round_bf16(v[j] + h8[j]);
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) val[i][j] = v[j];
+      for (int j = 0; j < 8; ++j) v[j] *= w[j];
     }
+    if (ln_b) {
+      float bb[8];
+      unpack8(reinterpret_cast<const u32x4*>(ln_b)[cc[i]], bb);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] += bb[j];
+    }
+    // every bf16 tensor of the separate ops is a rounding point: LayerNorm output, 1 + scale, the product,
+    // the sum; roundings go in pairs through one conversion
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) round_bf16_pair(v[j], v[j + 1]);
+    if (sc) {
+      float s8[8];
+      unpack8(sraw[i], s8);
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        float a = 1.0f + s8[j], b = 1.0f + s8[j + 1];
+        round_bf16_pair(a, b);
+        v[j] *= a;
+        v[j + 1] *= b;
+        round_bf16_pair(v[j], v[j + 1]);
+      }
+    }
+    if (sh) {
+      float h8[8];
+      unpack8(hraw[i], h8);
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        v[j] += h8[j];
+        v[j + 1] += h8[j + 1];
+        round_bf16_pair(v[j], v[j + 1]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) val[i][j] = v[j];
+  }
+  if (ragged) {  // slots past the end of the row: a zero cannot raise the row's absmax
+#pragma unroll
+    for (int i = 0; i < NCH; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) val[i][j] = ok[i] ? val[i][j] : 0.f;
   }
   if (!live) return;  // wave-uniform
   emit_row<NCH, TPR>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
@@ -184,44 +217,53 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const uint16_t* __res
   if (!live) row = rows - 1;
   const int nchunk = D >> 3;
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  // slots past the end of the row are clamped onto its last chunk: no load sits under a lane predicate
+  int cc[NCH];
+  bool ok[NCH];
+  u32x4 raw[NCH], wraw[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = t + i * TPR;
+    ok[i] = c < nchunk;
+    cc[i] = min(c, nchunk - 1);
+    raw[i] = xr[cc[i]];
+  }
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) wraw[i] = reinterpret_cast<const u32x4*>(w)[cc[i]];
   float val[NCH][8];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = t + i * TPR;
-    if (c < nchunk) {
-      unpack8(xr[c], val[i]);
+    unpack8(raw[i], val[i]);
+    float part = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) ss += val[i][j] * val[i][j];
-    }
+    for (int j = 0; j < 8; ++j) part += val[i][j] * val[i][j];
+    ss += ok[i] ? part : 0.f;
   }
   const float rrms = rsqrtf(row_sum<TPR>(ss, red) / (float)D + eps);
   if (!live) return;  // wave-uniform
   const float* rp = rope ? rope + (row / rows_per_batch) * rope_sb + (row % rows_per_batch) * 128 : nullptr;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
-    const int c = t + i * TPR;
-    if (c < nchunk) {
-      float wv[8];
-      unpack8(reinterpret_cast<const u32x4*>(w)[c], wv);
-      float v[8];
+    float wv[8];
+    unpack8(wraw[i], wv);
+    float v[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = round_bf16(round_bf16(val[i][j] * rrms) * wv[j]);
-      if (rp) {
-        const int off = (c * 8) & 127;  // offset inside the head: floats (cos, sin) of pairs off/2 .. off/2+3
-        const f32x4 t0 = *reinterpret_cast<const f32x4*>(rp + off);
-        const f32x4 t1 = *reinterpret_cast<const f32x4*>(rp + off + 4);
-        const float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+    for (int j = 0; j < 8; ++j) v[j] = round_bf16(round_bf16(val[i][j] * rrms) * wv[j]);
+    if (rp) {
+      const int off = (cc[i] * 8) & 127;  // offset inside the head: floats (cos, sin) of pairs off/2 .. off/2+3
+      const f32x4 t0 = *reinterpret_cast<const f32x4*>(rp + off);
+      const f32x4 t1 = *reinterpret_cast<const f32x4*>(rp + off + 4);
+      const float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const float cc = cs[2 * k], sn = cs[2 * k + 1];
-          const float x0 = v[2 * k], x1 = v[2 * k + 1];
-          v[2 * k] = mul_add_unfused(cc, x0, -sn, x1);
-          v[2 * k + 1] = mul_add_unfused(sn, x0, cc, x1);
-        }
+      for (int k = 0; k < 4; ++k) {
+        const float co = cs[2 * k], sn = cs[2 * k + 1];
+        const float x0 = v[2 * k], x1 = v[2 * k + 1];
+        v[2 * k] = mul_add_unfused(co, x0, -sn, x1);
+        v[2 * k + 1] = mul_add_unfused(sn, x0, co, x1);
       }
-      reinterpret_cast<u32x4*>(out + row * ldo)[c] = pack8(v);
     }
+    if (ok[i]) reinterpret_cast<u32x4*>(out + row * ldo)[cc[i]] = pack8(v);
   }
 }
 
@@ -241,19 +283,25 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restri
   const int nchunk = npre + (D >> 3);
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
   const u32x4* pr = reinterpret_cast<const u32x4*>(prefix + row * ldp);
+  // slots past the end of the row are clamped onto its last chunk: no load sits under a lane predicate
+  u32x4 raw[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = min(tid + i * 256, nchunk - 1);
+    raw[i] = __builtin_nontemporal_load(c < npre ? pr + c : xr + (c - npre));
+  }
   float val[NCH][8];
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = tid + i * 256;
-    if (c < nchunk) {
-      if (c < npre) {
-        unpack8(pr[c], val[i]);
-      } else {
-        u32x4 w = __builtin_nontemporal_load(xr + (c - npre));
-        unpack8(w, val[i]);
+    unpack8(raw[i], val[i]);
+    if (c >= npre) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(gelu_tanh_f32(val[i][j]));
-      }
+      for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(gelu_tanh_f32(val[i][j]));
+    }
+    if (c >= nchunk) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) val[i][j] = 0.f;  // keeps the row's absmax untouched
     }
   }
   emit_row<NCH, 256>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,

@@ -51,15 +51,15 @@ __global__ __launch_bounds__(256) void quant_rowwise_kernel(const uint16_t* __re
   if (row >= M) return;
   const int nchunk = K >> 3;
   const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  // slots past the end of the row are clamped onto its last chunk (a repeated chunk leaves the absmax as it
+  // is), so that no load sits under a lane predicate and the row's loads are issued back to back
   u32x4 cache[NCH];
   float amax = 0.f;
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    int c = lane + i * 64;
-    if (c < nchunk) {
-      cache[i] = __builtin_nontemporal_load(xr + c);
-      if (SCALED) amax = fmaxf(amax, absmax_bf16x8(cache[i]));
-    }
+  for (int i = 0; i < NCH; ++i) cache[i] = __builtin_nontemporal_load(xr + min(lane + i * 64, nchunk - 1));
+  if (SCALED) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) amax = fmaxf(amax, absmax_bf16x8(cache[i]));
   }
   float inv = 1.0f;
   if (SCALED) {

@@ -220,8 +220,16 @@ class FluxDiTRunner:
         nw = self.norm_w
         qkv_a = qkv_a.view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         qkv_b = qkv_b.view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
-        o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
-        o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
+        # With one batch entry the text and image rows of an intermediate share one [text; image] buffer, so
+        # that the row kernels between the GEMM pairs (quantise, GELU) run once over both streams; with more
+        # entries the rows of one stream would not be evenly strided for the GEMM.
+        joint = B == 1
+        if joint:
+            o = torch.empty((1, St + Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
+            o_b, o_a = o[:, :St], o[:, St:]
+        else:
+            o_b = torch.empty((B, St, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
+            o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         qb_, kb_, vb_ = qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:]
         qa_, ka_, va_ = qkv_a[:, :HEADS], qkv_a[:, HEADS:2 * HEADS], qkv_a[:, 2 * HEADS:]
         # joint attention over [text; image] rows with the per-stream q/k RMSNorm weights and the RoPE table
@@ -234,16 +242,29 @@ class FluxDiTRunner:
         # gated residual, LN-modulate, MLP + gated residual.  Each pair of linears goes out as one grouped
         # submission so that the 512-token text problem runs beside the image problem instead of after it.
         xa, xb = img.reshape(B * Si, d), txt.reshape(B * St, d)
-        qa, sa = ops.quantize_fp8(o_a.view(B * Si, d), scaled=self.scaled)
-        qb, sb = ops.quantize_fp8(o_b.view(B * St, d), scaled=self.scaled)
+        if joint:
+            qo, so = ops.quantize_fp8(o.view(St + Si, d), scaled=self.scaled)
+            qb, qa = qo[:St], qo[St:]
+            sb, sa = (so[:St], so[St:]) if so is not None else (None, None)
+        else:
+            qa, sa = ops.quantize_fp8(o_a.view(B * Si, d), scaled=self.scaled)
+            qb, sb = ops.quantize_fp8(o_b.view(B * St, d), scaled=self.scaled)
         xa, xb = _gemm_pair(L[pre + "attn.a_to_out"], dict(a_q=qa, a_s=sa, resid=xa, gate=ma[2], rows_per_batch=Si),
                             L[pre + "attn.b_to_out"], dict(a_q=qb, a_s=sb, resid=xb, gate=mb[2], rows_per_batch=St))
         qa, sa = self._modulate_q(xa.view(B, Si, d), ma[4], ma[3])
         qb, sb = self._modulate_q(xb.view(B, St, d), mb[4], mb[3])
-        ha, hb = _gemm_pair(L[pre + "ff_a.0"], dict(a_q=qa.view(-1, d), a_s=sa),
-                            L[pre + "ff_b.0"], dict(a_q=qb.view(-1, d), a_s=sb))
-        qa, sa = self._gelu_q(ha)
-        qb, sb = self._gelu_q(hb)
+        if joint:
+            h = torch.empty((St + Si, L[pre + "ff_a.0"].n), dtype=torch.bfloat16, device=img.device)
+            _gemm_pair(L[pre + "ff_a.0"], dict(a_q=qa.view(-1, d), a_s=sa, out=h[St:]),
+                       L[pre + "ff_b.0"], dict(a_q=qb.view(-1, d), a_s=sb, out=h[:St]))
+            qh, sh_ = self._gelu_q(h)
+            qb, qa = qh[:St], qh[St:]
+            sb, sa = (sh_[:St], sh_[St:]) if sh_ is not None else (None, None)
+        else:
+            ha, hb = _gemm_pair(L[pre + "ff_a.0"], dict(a_q=qa.view(-1, d), a_s=sa),
+                                L[pre + "ff_b.0"], dict(a_q=qb.view(-1, d), a_s=sb))
+            qa, sa = self._gelu_q(ha)
+            qb, sb = self._gelu_q(hb)
         xa, xb = _gemm_pair(L[pre + "ff_a.2"], dict(a_q=qa, a_s=sa, resid=xa, gate=ma[5], rows_per_batch=Si),
                             L[pre + "ff_b.2"], dict(a_q=qb, a_s=sb, resid=xb, gate=mb[5], rows_per_batch=St))
         return xa.view(B, Si, d), xb.view(B, St, d)
