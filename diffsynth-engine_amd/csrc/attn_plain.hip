@@ -364,15 +364,22 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
   // operand.  The row sum adds the fp32 values with plain v_add_f32 (v_dot2c_f32_bf16 on the packed pair
   // would be one instruction, but it executes on the matrix pipe and was measured to cost a third of the
   // MFMA rate).
+  // Each result is pinned where it is computed by an empty volatile asm that "uses" it: the exponential, the
+  // convert and the add are pure, and the optimiser otherwise sinks them to the block of their first use (the
+  // PV MFMAs behind the next branch, the row sum at the end of the interval), past the scheduling barriers:
+  // the MFMA slots they were written into then run bare and the VALU work runs in MFMA-free clumps.
   float p_even = 0.f, lsum0 = 0.f, lsum1 = 0.f;
   auto exp_entry = [&](const f32x16 (&s)[2], uint32_t (&pw)[2][8], int e) {
-    const float pv = __builtin_amdgcn_exp2f(s[e >> 4][e & 15]);
+    float pv = __builtin_amdgcn_exp2f(s[e >> 4][e & 15]);
     if (e & 1) {
-      pw[e >> 4][(e & 15) >> 1] = pack_bf16x2(p_even, pv);
+      uint32_t w = pack_bf16x2(p_even, pv);
       lsum1 += pv;
+      asm volatile("" : "+v"(w), "+v"(lsum1));
+      pw[e >> 4][(e & 15) >> 1] = w;
     } else {
-      p_even = pv;
       lsum0 += pv;
+      asm volatile("" : "+v"(pv), "+v"(lsum0));
+      p_even = pv;
     }
   };
   auto qk = [&](f32x16 (&s)[2], int stage) {
