@@ -227,6 +227,10 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
   }
   // rows are handled eight at a time so that the residual loads of a group are in flight together;
   // interior tiles (the common case) run without per-row bounds tests
+  // row pointers: one 64-bit multiply per lane, then a uniform stride of four rows per step
+  uint16_t* const out_lane = p.out + (int64_t)(m_base + r0) * p.ldo + n;
+  const uint16_t* const res_lane = RESID ? p.resid + (int64_t)(m_base + r0) * p.ldr + n : nullptr;
+  const int64_t out_step = 4 * p.ldo, res_step = 4 * p.ldr;
   auto rows8 = [&](int it0, bool guarded) {
     u32x4 v[8], rv[8];
     bool ok[8];
@@ -236,7 +240,7 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
       const int m = m_base + ml;
       ok[u] = !guarded || (m < p.M && col_ok);
       v[u] = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
-      if (RESID && ok[u]) rv[u] = *reinterpret_cast<const u32x4*>(p.resid + (int64_t)m * p.ldr + n);
+      if (RESID && ok[u]) rv[u] = *reinterpret_cast<const u32x4*>(res_lane + (it0 + u) * res_step);
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -254,7 +258,7 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
           v[u][c] = pack_bf16x2(bf16_lo(rv[u][c]) + t0, bf16_hi(rv[u][c]) + t1);
         }
       }
-      *reinterpret_cast<u32x4*>(p.out + (int64_t)m * p.ldo + n) = v[u];
+      *reinterpret_cast<u32x4*>(out_lane + (it0 + u) * out_step) = v[u];
     }
   };
   const bool interior = m_base + 128 <= p.M && n_base + 128 <= p.N;  // wave-uniform
