@@ -179,7 +179,7 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
     const int k0 = kb * KB;
     const int lo = k0 >= skv0 ? 1 : 0, hi = k0 + KB - 1 >= skv0 ? 1 : 0;
     const bool simple = lo == hi && k0 + KB <= skv_all;
-    if (simple && ptr_seg == lo) {
+    if (__builtin_expect(simple && ptr_seg == lo, 1)) {
       const int64_t ks = lo ? kstep[1] : kstep[0], vs = lo ? vstep[1] : vstep[0];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -308,13 +308,13 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
   auto interval_head = [&](int kb) {
     __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4): only block kb+2 may still be in flight
     __builtin_amdgcn_s_barrier();
-    if (kb + 3 < kb_end) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
+    if (__builtin_expect(kb + 3 < kb_end, 1)) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
   };
   // Softmax reference.  mask_tail masks the ragged tail of block `blk`; ref_scan subtracts the current
   // reference and returns the block maximum of the lane's query; ref_move shifts the reference (rescaling O and l), which
   // is needed only when a block maximum leaves the safe range.
   auto mask_tail = [&](f32x16 (&s)[2], int blk) {
-    if ((blk + 1) * KB > skv_all) {  // ragged tail of the key axis
+    if (__builtin_expect((blk + 1) * KB > skv_all, 0)) {  // ragged tail of the key axis
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
     }
   };
   auto ref_scan = [&](f32x16 (&s)[2], int blk) -> float {
-    if (any_ref) {
+    if (__builtin_expect(any_ref, 0)) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -456,10 +456,10 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
       pv_slot(j);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (kb + 1 < kb_end) {
+    if (__builtin_expect(kb + 1 < kb_end, 1)) {
       mask_tail(s_next, kb + 1);
       const float mx = SCAN ? ref_scan(s_next, kb + 1) : 0.f;
-      if (SCAN && ref_must_move(mx, kb + 1)) {
+      if (SCAN && __builtin_expect(ref_must_move(mx, kb + 1), 0)) {
         // rare: O, l and the scores of block kb+1 move to the new reference now; the part of P(kb) that
         // the remaining PV MFMAs still have to accumulate follows (one more bf16 rounding on it)
         const float alpha = ref_move(s_next, mx, kb + 1);
