@@ -45,3 +45,29 @@ def test_graph_refuses_host_inputs(dev):
 
     with pytest.raises(RuntimeError):
         GraphedStep(lambda **kw: None, x=torch.zeros(4))
+
+
+def test_wan_step_graph_replays_equal_eager(dev):
+    from oracle import wan as ow
+
+    from diffsynth_engine_amd.graph import GraphedStep
+    from diffsynth_engine_amd.wan_dit import WanDiTRunner
+
+    cfg = dict(ow.config_14b(), dim=512, ffn_dim=1024, num_heads=4, num_layers=2)
+    sd = ow.init_params(cfg, dtype=torch.bfloat16, seed=1, bias_std=0.02)
+    runner = WanDiTRunner(sd, cfg, scaled=True, device=dev)
+
+    def inputs(seed):
+        g = torch.Generator().manual_seed(seed)
+        return dict(x=torch.randn(1, 16, 2, 12, 16, generator=g).bfloat16().to(dev),
+                    context=torch.randn(1, 32, 4096, generator=g).bfloat16().to(dev),
+                    timestep=torch.tensor([float(200 + 100 * seed)], device=dev).bfloat16())
+
+    step = GraphedStep(runner, **inputs(0))
+    for r in range(1, 4):
+        inp = inputs(r)
+        eager = runner(**inp).clone()
+        torch.cuda.synchronize()
+        got = step(**inp).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), r
