@@ -213,12 +213,13 @@ class GemmTimer:
         return len(self.records), flops, secs
 
 
-def time_kernel(torch, fn, args_list=None, reps=5):
+def time_kernel(torch, fn, args_list=None, reps=10):
     """Seconds per call of ``fn`` with the host taken out of the measurement: the calls are recorded into one HIP
     graph and the graph is replayed, so a 6 us kernel is not reported at the 12 us it takes Python to launch it.
     ``args_list``: one argument tuple per call of the recorded sequence; bandwidth-bound kernels get a rotation of
     buffers larger than the 256 MB Infinity Cache so that every call reads HBM.  Without it ``fn()`` is recorded
-    ten times on the same operands (matrix kernels: the caches are left as they are)."""
+    ten times on the same operands (matrix kernels: the caches are left as they are).  At least 100 calls are
+    timed (``reps`` replays); the figure is their mean."""
     calls = [()] * 10 if args_list is None else list(args_list)
     for a in calls[:3]:
         fn(*a)
@@ -227,6 +228,7 @@ def time_kernel(torch, fn, args_list=None, reps=5):
     with torch.cuda.graph(graph):
         for a in calls:
             fn(*a)
+    graph.replay()  # warm-up: with the three eager calls above, at least 20 calls before the timed ones
     graph.replay()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
