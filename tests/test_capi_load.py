@@ -152,3 +152,14 @@ def test_attention_workspace_size_query():
     P.head_dim = 64
     assert lib.dsx_attn_workspace_bytes(P) == 0
     assert lib.dsx_attn_workspace_bytes(None) == 0
+
+
+def test_graphed_step_refuses_host_inputs():
+    """A host tensor cannot be an input of a recorded step (its copy to the device cannot be recorded): refused
+    before anything touches the GPU."""
+    import torch
+
+    from diffsynth_engine_amd.graph import GraphedStep
+
+    with pytest.raises(RuntimeError):
+        GraphedStep(lambda **kw: None, x=torch.zeros(4))
