@@ -9,10 +9,10 @@
 // lane (g, j) then holds ONE token m = j and four consecutive output features per register
 // quad, so the per-token scale is a per-lane constant and the bf16 results leave as 8-byte stores.
 //
-// Main kernel: 256x256 output tile per workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
-// tiles (256 fp32 accumulators).  Operands reach LDS by global_load_lds_dwordx4 (HBM/L2 -> LDS
-// without staging registers) in 128-byte-wide units through a five-slot ring; MFMA operand
-// fragments are double-buffered in registers so that LDS reads overlap the MFMAs.  LDS rows are
+// Main kernel: 256x256 output tile per workgroup, 8 waves as 2x4, each wave 128x64 = 4x2 MFMA
+// tiles (128 fp32 accumulators), two waves per SIMD.  Operands reach LDS by global_load_lds_dwordx4
+// (HBM/L2 -> LDS without staging registers) in 128-byte-wide units through a five-slot ring; MFMA
+// operand fragments are read one step ahead so that LDS reads overlap the MFMAs.  LDS rows are
 // 128 B (8 chunks of 16 B); chunk c of row r lives at chunk c ^ ((r/2)&7), which makes 16 lanes
 // reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
 // One launch can carry two independent problems (the image- and text-stream linears of a joint
@@ -155,43 +155,48 @@ __device__ __forceinline__ void store_ct(const GemmArgs& p, f32x16 (&acc)[4][4],
   }
 }
 
-// LDS-staged store of a wave's 128 (m) x 128 (n) block: the C^T accumulators are scaled, biased,
-// rounded to bf16 and written to a wave-private LDS region as [m][n] rows (272-byte pitch: 256 data
-// bytes + 16 pad, so 8-byte column writes of 32 consecutive rows spread over the banks), then read
-// back as 16-byte chunks along n so that 16 lanes emit one contiguous 256-byte row segment.
+// LDS-staged store of a wave's 64 (m) x 128 (n) block: the C^T accumulators are scaled, biased, rounded to
+// bf16 and written to a wave-private LDS region as [m][n] rows (272-byte pitch: 256 data bytes + 16 pad, so
+// 8-byte column writes of 32 consecutive rows spread over the banks), then read back as 16-byte chunks
+// along n so that 16 lanes emit one contiguous 256-byte row segment.
 constexpr int kEpiPitch = 272;
-constexpr int kEpiBytesPerWave = 128 * kEpiPitch;  // 34 816
 constexpr int kMainLdsBytes = 160 * 1024;  // five operand stages; the epilogue staging (136 KiB) reuses them
 
-// Per-lane epilogue operands, fetched in one batch so that their latency is paid once.
-struct EpiOperands {
-  u32x2 bias[4][4];  // [tn][rq]: 4 consecutive bf16 at n = tn*32 + 8*rq + 4*g
-  float sc[4];       // [tm]: a_scale[m] * w_scale
-};
-__device__ __forceinline__ void load_epi_operands(const GemmArgs& p, EpiOperands& e, int n_base,
-                                                  int m_base, int lane) {
-  const int g = lane >> 5, li = lane & 31;
-  const float ws = p.w_scale ? *p.w_scale : 1.0f;
-#pragma unroll
-  for (int tn = 0; tn < 4; ++tn)
-#pragma unroll
-    for (int rq = 0; rq < 4; ++rq) {
-      const int n = n_base + tn * 32 + 8 * rq + 4 * g;
-      e.bias[tn][rq] = (p.bias && n < p.N) ? *reinterpret_cast<const u32x2*>(p.bias + n) : u32x2{0, 0};
-    }
-#pragma unroll
-  for (int tm = 0; tm < 4; ++tm) {
-    const int m = m_base + tm * 32 + li;
-    e.sc[tm] = (p.a_scale && m < p.M ? p.a_scale[m] : 1.0f) * ws;
-  }
+constexpr int SK = 64;                   // K bytes per MFMA step
+constexpr int UK = 128;                  // K bytes per unit row
+constexpr int NSLOT = 5;
+constexpr int kUnitBytes = 256 * UK;     // 32 KiB
+
+// 128-byte rows: 16-byte chunk c of row r lives at chunk c ^ ((r/2)&7); two rows span the 64 banks.
+__device__ __forceinline__ int unit_off(int row, int chunk) {
+  return row * UK + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
+// ------------------------------------------------------------------------------------------
+// Main kernel: K % 128 == 0.  Operands move HBM -> LDS in units of one operand x 128 bytes of K
+// (256 rows x 128 B = 32 KiB), so that every async load instruction (64 lanes x 16 B) fetches
+// eight whole 128-byte cache lines: with 64-byte rows each line would be requested twice, a step
+// apart, and the second request stalls the L1 behind the still-pending first one.  Five unit
+// slots (160 KiB) form a ring W0 A0 W1 A1 W2 | A2 W3 ...; one MFMA step consumes 64 bytes of K,
+// i.e. half of a W unit and half of an A unit.
+// Eight waves as 2 (n) x 4 (m), each 128 (n) x 64 (m) = 4x2 MFMA tiles (128 accumulators), so that two
+// waves share a SIMD: while one waits at the step's barrier or for its operands, the other's MFMAs keep
+// the matrix pipe busy, and the two overlap their epilogues.  (Four waves of 128 x 128 read a third
+// fewer fragment bytes per MFMA but leave the pipe idle in those waits: 3-12 % slower.)
+// ------------------------------------------------------------------------------------------
+constexpr int kEpiBytesPerWave = 64 * kEpiPitch;  // 17 408; eight of them fit the operand stages
+
+struct EpiOperands {
+  u32x2 bias[4][4];  // [tn][rq]: 4 consecutive bf16 at n = tn*32 + 8*rq + 4*g
+  float sc[2];       // [tm]: a_scale[m] * w_scale
+};
+
 template <bool RESID>
-__device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][4], const EpiOperands& e,
-                                             uint8_t* wave_lds, int n_base, int m_base, int lane) {
+__device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][2], const EpiOperands& e,
+                                              uint8_t* wave_lds, int n_base, int m_base, int lane) {
   const int g = lane >> 5, li = lane & 31;
 #pragma unroll
-  for (int tm = 0; tm < 4; ++tm) {
+  for (int tm = 0; tm < 2; ++tm) {
     const float sc = e.sc[tm];
     uint8_t* lrow = wave_lds + (tm * 32 + li) * kEpiPitch;
 #pragma unroll
@@ -209,25 +214,19 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
       }
     }
   }
-  // the region is private to this wave: its own LDS writes only have to have completed
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the region is private to this wave
   __builtin_amdgcn_wave_barrier();
   const int ch = lane & 15, r0 = lane >> 4;
   const int n = n_base + ch * 8;
   const bool col_ok = n < p.N;
-  // The gate is one vector per batch element: when the wave's 128 rows lie in one batch element (always,
-  // unless a tile straddles two) it is fetched once, and the row -> batch division leaves the row loop.
   u32x4 gv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
   bool gate_per_row = false;
   const bool gated = RESID && p.gate != nullptr;
   if (gated) {
-    const int b_lo = m_base / p.rows_per_batch, b_hi = min(m_base + 127, p.M - 1) / p.rows_per_batch;
+    const int b_lo = m_base / p.rows_per_batch, b_hi = min(m_base + 63, p.M - 1) / p.rows_per_batch;
     gate_per_row = b_lo != b_hi;
     if (!gate_per_row && col_ok) gv = *reinterpret_cast<const u32x4*>(p.gate + (int64_t)b_lo * p.gate_sb + n);
   }
-  // rows are handled eight at a time so that the residual loads of a group are in flight together;
-  // interior tiles (the common case) run without per-row bounds tests
-  // row pointers: one 64-bit multiply per lane, then a uniform stride of four rows per step
   uint16_t* const out_lane = p.out + (int64_t)(m_base + r0) * p.ldo + n;
   const uint16_t* const res_lane = RESID ? p.resid + (int64_t)(m_base + r0) * p.ldr + n : nullptr;
   const int64_t out_step = 4 * p.ldo, res_step = 4 * p.ldr;
@@ -250,7 +249,6 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
         u32x4 gu = gv;
         if (gate_per_row)
           gu = *reinterpret_cast<const u32x4*>(p.gate + (int64_t)(m / p.rows_per_batch) * p.gate_sb + n);
-        // rounding points of the separate ops: bf16(gate * proj), then bf16(resid + .)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           const float t0 = gated ? round_bf16(bf16_lo(gu[c]) * bf16_lo(v[u][c])) : bf16_lo(v[u][c]);
@@ -261,36 +259,18 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
       *reinterpret_cast<u32x4*>(out_lane + (it0 + u) * out_step) = v[u];
     }
   };
-  const bool interior = m_base + 128 <= p.M && n_base + 128 <= p.N;  // wave-uniform
+  const bool interior = m_base + 64 <= p.M && n_base + 128 <= p.N;  // wave-uniform
   if (interior) {
 #pragma unroll
-    for (int it0 = 0; it0 < 32; it0 += 8) rows8(it0, false);
+    for (int it0 = 0; it0 < 16; it0 += 8) rows8(it0, false);
   } else {
 #pragma unroll
-    for (int it0 = 0; it0 < 32; it0 += 8) rows8(it0, true);
+    for (int it0 = 0; it0 < 16; it0 += 8) rows8(it0, true);
   }
 }
 
-// ------------------------------------------------------------------------------------------
-// Main kernel: K % 128 == 0.  Operands move HBM -> LDS in units of one operand x 128 bytes of K
-// (256 rows x 128 B = 32 KiB), so that every async load instruction (64 lanes x 16 B) fetches
-// eight whole 128-byte cache lines: with 64-byte rows each line would be requested twice, a step
-// apart, and the second request stalls the L1 behind the still-pending first one.  Five unit
-// slots (160 KiB) form a ring W0 A0 W1 A1 W2 | A2 W3 ...; one MFMA step consumes 64 bytes of K,
-// i.e. half of a W unit and half of an A unit.
-// ------------------------------------------------------------------------------------------
-constexpr int SK = 64;                   // K bytes per MFMA step
-constexpr int UK = 128;                  // K bytes per unit row
-constexpr int NSLOT = 5;
-constexpr int kUnitBytes = 256 * UK;     // 32 KiB
-
-// 128-byte rows: 16-byte chunk c of row r lives at chunk c ^ ((r/2)&7); two rows span the 64 banks.
-__device__ __forceinline__ int unit_off(int row, int chunk) {
-  return row * UK + ((chunk ^ ((row >> 1) & 7)) << 4);
-}
-
 template <bool RESID>
-__global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmPair q) {
+__global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   int L = logical_tile(blockIdx.x, q.total);
   if (L >= q.total) return;
@@ -302,116 +282,154 @@ __global__ __launch_bounds__(256) void fp8_gemm_kernel(GemmPair q) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wn = wave >> 1, wm = wave & 1;
+  const int wave = tid >> 6;            // 0..7
+  const int wn = wave >> 2, wm = wave & 3;
   const int g = lane >> 5, li = lane & 31;
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // ---- async loads: one wave instruction fills 1 KiB of LDS = 8 rows x 128 B; lane l lands at
-  //      row l/8, physical chunk l%8, so it fetches logical chunk (l%8) ^ swz(row).
-  //      Per unit a wave issues 8 instructions for its 64 rows.
+  // async loads: per unit a wave issues 4 instructions for its 32 rows
   const int ld_r = lane >> 3, ld_p = lane & 7;
-  uint32_t w_off[8], a_off[8];
+  uint32_t w_off[4], a_off[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = (wave * 8 + i) * 8 + ld_r;
+  for (int i = 0; i < 4; ++i) {
+    const int row = (wave * 4 + i) * 8 + ld_r;
     const int c = ld_p ^ ((row >> 1) & 7);
     w_off[i] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.ldw + c * 16;
     a_off[i] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.lda + c * 16;
   }
   const uint8_t* w_base = p.w + (int64_t)n0 * p.ldw;
   const uint8_t* a_base = p.a + (int64_t)m0 * p.lda;
-  const int nk = p.K / SK;       // MFMA steps, even
-  const int nu = nk / 2;         // units per operand
-  // unit (j, op): op 0 = W, 1 = A; ring slot (2j + op) % 5
+  const int nk = p.K / SK;
+  const int nu = nk / 2;
+  // The async loads are issued as assembly in the scalar-base + 32-bit-lane-offset form: the builtin takes a
+  // 64-bit per-lane address, and eight of those (plus their increments) are sixteen registers this kernel,
+  // at 256 per wave, does not have.  M0 carries the LDS destination; nothing else here uses M0.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
   auto issue_load = [&](int j, int op, int i) {
     const int slot = (2 * j + op) % NSLOT;
-    j = min(j, nu - 1);  // past the end: re-fetch the last unit into a slot nobody reads again
-    uint8_t* dst = smem + slot * kUnitBytes + (wave * 8 + i) * 1024;
-    const uint8_t* src = (op ? a_base + a_off[i] : w_base + w_off[i]) + (int64_t)j * UK;
-    __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
+    j = min(j, nu - 1);
+    const uint32_t dst = lds0 + slot * kUnitBytes + (wave_u * 4 + i) * 1024;
+    const uint8_t* ub = (op ? a_base : w_base) + (int64_t)j * UK;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(op ? a_off[i] : w_off[i]), "s"(ub), "s"(dst)
+                 : "memory", "m0");
   };
+#pragma clang diagnostic pop
 
-  // ---- fragments: 4 W tiles + 4 A tiles, two 16-byte halves each = 16 LDS reads per step
+  // Fragments: 4 W tiles + 2 A tiles, two 16-byte halves each = 12 LDS reads per step.  W tile i feeds MFMAs
+  // 2i and 2i+1 only, so the next step's W tile i is read into the SAME registers right after MFMA 2i+1 (seven
+  // MFMAs before its use); only the A fragments, which every MFMA of a step reads, are double-buffered.  That
+  // is 64 fragment registers instead of 96, which is what lets 128 accumulators fit in 256 registers.
   const int w_row = wn * 128 + li;
-  const int a_row = wm * 128 + li;
-  struct Frags {
-    i32x4 w[4][2];
-    i32x4 a[4][2];
+  const int a_row = wm * 64 + li;
+  i32x4 fw[4][2];
+  i32x4 fa[2][2][2];  // [buffer][tile][half]
+  // read addresses: one lane constant per (step parity, half) and operand; the tile adds 32 rows = 4096 bytes
+  // (the swizzle of row + 32t equals that of row) and the ring slot adds a scalar
+  uint32_t w_la[2][2], a_la[2][2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      w_la[par][half] = (uint32_t)unit_off(w_row, par * 4 + g * 2 + half);
+      a_la[par][half] = (uint32_t)unit_off(a_row, par * 4 + g * 2 + half);
+    }
+  auto read_w = [&](int j, int par, int t, int half) {   // W fragment (tile t) of MFMA step 2j + par
+    uint32_t slot_off = (uint32_t)(((2 * j) % NSLOT) * kUnitBytes);
+    asm volatile("" : "+s"(slot_off));  // added at the read, from a scalar: not a register per combination
+    fw[t][half] = *reinterpret_cast<const i32x4*>(smem + (slot_off + w_la[par][half]) + t * 4096);
   };
-  auto read_frag = [&](Frags& f, int j, int par, int idx) {   // fragments of MFMA step 2j + par
-    const uint8_t* sW = smem + ((2 * j) % NSLOT) * kUnitBytes;
-    const uint8_t* sA = smem + ((2 * j + 1) % NSLOT) * kUnitBytes;
-    const int t = idx >> 2, half = idx & 1, is_a = (idx >> 1) & 1;
-    const int c = par * 4 + g * 2 + half;
-    if (is_a)
-      f.a[t][half] = *reinterpret_cast<const i32x4*>(sA + unit_off(a_row + t * 32, c));
-    else
-      f.w[t][half] = *reinterpret_cast<const i32x4*>(sW + unit_off(w_row + t * 32, c));
+  auto read_a = [&](int buf, int j, int par, int t, int half) {
+    uint32_t slot_off = (uint32_t)(((2 * j + 1) % NSLOT) * kUnitBytes);
+    asm volatile("" : "+s"(slot_off));
+    fa[buf][t][half] = *reinterpret_cast<const i32x4*>(smem + (slot_off + a_la[par][half]) + t * 4096);
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  auto mfma_one = [&](const Frags& f, int idx) {
-    const int i = idx >> 2, j = idx & 3;
-    const i32x8 fw = {f.w[i][0].x, f.w[i][0].y, f.w[i][0].z, f.w[i][0].w,
-                      f.w[i][1].x, f.w[i][1].y, f.w[i][1].z, f.w[i][1].w};
-    const i32x8 fa = {f.a[j][0].x, f.a[j][0].y, f.a[j][0].z, f.a[j][0].w,
-                      f.a[j][1].x, f.a[j][1].y, f.a[j][1].z, f.a[j][1].w};
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fw, fa, acc[i][j], 0, 0, 0, 0, 0, 0);
+  auto mfma_one = [&](int buf, int idx) {   // idx 0..7: W tile idx/2, A tile idx%2
+    const int i = idx >> 1, j = idx & 1;
+    const i32x8 vw = {fw[i][0].x, fw[i][0].y, fw[i][0].z, fw[i][0].w, fw[i][1].x, fw[i][1].y, fw[i][1].z, fw[i][1].w};
+    const i32x8 va = {fa[buf][j][0].x, fa[buf][j][0].y, fa[buf][j][0].z, fa[buf][j][0].w,
+                      fa[buf][j][1].x, fa[buf][j][1].y, fa[buf][j][1].z, fa[buf][j][1].w};
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vw, va, acc[i][j], 0, 0, 0, 0, 0, 0);
   };
 
-  // Step s multiplies the fragments of step s (in registers, fc) while reading those of step s+1.
-  // Even step 2j: its reads stay inside units j, already known to have landed; no barrier.  It
-  //   issues the loads of W unit j+2 into the slot A unit j-1 left at the last barrier.
-  // Odd step 2j+1: its reads open units j+1, so first wait until only the 8 newest loads (W unit
-  //   j+2) are in flight, then the barrier; that barrier also says every wave has read W unit j
-  //   for the last time, whose slot takes the loads of A unit j+2.
-  // 16 MFMAs, each followed by one LDS read and, for the first eight, one async load;
-  // sched_barrier pins that order.
-  auto step = [&](int j, int par, const Frags& fc, Frags& fn) {   // MFMA step 2j + par; par is a literal
+  // as in fp8_gemm_kernel, with 8 MFMAs, 12 fragment reads and 4 async loads per wave and step; the
+  // fragments of step 2j + par sit in fw and fa[par]
+  auto step = [&](int j, int par) {
     if (par) {
-      __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
+      __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
     } else {
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
     }
 #pragma unroll
-    for (int idx = 0; idx < 16; ++idx) {
-      mfma_one(fc, idx);
-      read_frag(fn, j + par, par ^ 1, idx);
-      if (idx < 8) issue_load(j + 2, par, idx);
+    for (int idx = 0; idx < 8; ++idx) {
+      mfma_one(par, idx);
+      if (idx & 1) {  // W tile idx/2 has been read for the last time in this step
+        read_w(j + par, par ^ 1, idx >> 1, 0);
+        read_w(j + par, par ^ 1, idx >> 1, 1);
+      } else {
+        read_a(par ^ 1, j + par, par ^ 1, idx >> 2, (idx >> 1) & 1);
+        issue_load(j + 2, par, idx >> 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  Frags f0, f1;
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) issue_load(u >> 1, u & 1, i);
-  __builtin_amdgcn_s_waitcnt(0x4f70);  // vmcnt(16): W and A unit 0 have landed
+    for (int i = 0; i < 4; ++i) issue_load(u >> 1, u & 1, i);
+  __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): W and A unit 0 have landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int idx = 0; idx < 16; ++idx) read_frag(f0, 0, 0, idx);
+  for (int t = 0; t < 4; ++t) {
+    read_w(0, 0, t, 0);
+    read_w(0, 0, t, 1);
+  }
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    read_a(0, 0, 0, t, 0);
+    read_a(0, 0, 0, t, 1);
+  }
 
   for (int j = 0; j < nu; ++j) {
-    step(j, 0, f0, f1);
-    step(j, 1, f1, f0);
+    step(j, 0);
+    step(j, 1);
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is reused
 
-  // (the launcher sends shapes the vectorised epilogue cannot store to the generic kernel)
   EpiOperands epi;
-  load_epi_operands(p, epi, n0 + wn * 128, m0 + wm * 128, lane);
+  {
+    const float ws = p.w_scale ? *p.w_scale : 1.0f;
+    const int n_base = n0 + wn * 128, m_base = m0 + wm * 64;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        const int n = n_base + t * 32 + 8 * rq + 4 * g;
+        epi.bias[t][rq] = (p.bias && n < p.N) ? *reinterpret_cast<const u32x2*>(p.bias + n) : u32x2{0, 0};
+      }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int m = m_base + t * 32 + li;
+      epi.sc[t] = (p.a_scale && m < p.M ? p.a_scale[m] : 1.0f) * ws;
+    }
+  }
   __syncthreads();  // every wave is done reading the operand stages
-  store_ct_lds<RESID>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 128, lane);
+  store_ct_lds<RESID>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 64, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -606,9 +624,9 @@ static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStre
   q.total = q.total0 + (p1 ? p1->tiles_m * p1->tiles_n : 0);
   const int grid = ((q.total + 7) / 8) * 8;
   if (p0.resid)
-    fp8_gemm_kernel<true><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<true><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   else
-    fp8_gemm_kernel<false><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
