@@ -70,3 +70,30 @@ def test_small_model_step(dev):
     c = _cos(got, want)
     # same criterion as the Flux step: as close to the oracle as the oracle is to itself across torch backends
     assert c >= 0.99 and c >= min(0.999, _cos(want, want_dev) - 0.002), (c, _cos(want, want_dev))
+
+
+def test_two_layers_at_the_14b_width(dev):
+    """Wan2.1-14B's own width (5120 = 40 heads x 128, FFN 13824, 512 text tokens) on two layers and a
+    5 x 60 x 104 latent = 7800 video tokens, oracle evaluated by torch on the device with the same weights.
+    Same criterion as the full-depth Flux step: the oracle run again with the lowest mantissa bit of every
+    1024th latent element flipped is the yardstick for how far two correct evaluations of the scaled-fp8 step
+    may lie apart."""
+    from bench import wan_state_dict_stream
+    from diffsynth_engine_amd.wan_dit import WanDiTRunner
+
+    cfg = dict(ow.config_14b(), num_layers=2)
+    sd = dict(wan_state_dict_stream(cfg, dev, seed=0))
+    g = torch.Generator(device=dev).manual_seed(4)
+    x = torch.randn(1, 16, 5, 60, 104, generator=g, device=dev).bfloat16()
+    ctx = torch.randn(1, 512, 4096, generator=g, device=dev).bfloat16()
+    t = torch.tensor([500.0], device=dev).bfloat16()
+    got = WanDiTRunner(sd, cfg, scaled=True, device=dev)(x, ctx, t)
+    assert torch.isfinite(got.float()).all()
+    P = ow.Params(sd, "fp8_scaled")
+    want = ow.wan_dit_forward(P, x, ctx, t, cfg)
+    nudged = x.clone()
+    nudged.view(torch.int16).flatten()[::1024] ^= 1
+    want_nudged = ow.wan_dit_forward(P, nudged, ctx, t, cfg)
+    assert got.shape == want.shape
+    c, floor = _cos(got, want), _cos(want, want_nudged)
+    assert c >= 0.99 and c >= min(0.999, floor - 1e-3), (c, floor)
