@@ -100,6 +100,41 @@ def test_full_size_attention_invariants(dev):
     assert err <= 2e-2, err
 
 
+def test_wan_size_attention_through_its_seam(dev):
+    """Wan2.1-14B's calls at their real shapes through `wan_attention` ((B, S, H*D) in and out, wan_dit.py:18-22):
+    self-attention over 32 760 tokens (a ragged last key block: 32 760 = 511 x 64 + 56) and cross-attention to
+    512 text tokens, 40 heads.  Constant V comes back unchanged; sampled query rows of three heads agree with
+    torch's fp32 SDPA on the device."""
+    from diffsynth_engine_amd.attention import wan_attention
+
+    H, S, D = 40, 32760, 128
+    g = torch.Generator(device=dev).manual_seed(13)
+    q, k, v = [torch.randn(1, S, H * D, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(3)]
+    rows = torch.tensor([0, 31, 255, 256, 16383, 32703, 32704, 32759], device=dev)
+    heads = (0, 17, 39)
+
+    def sampled_ref(k_, v_):
+        hs = lambda t, h: t[:, :, h * D:(h + 1) * D].float()
+        return torch.stack([torch.nn.functional.scaled_dot_product_attention(
+            hs(q, h)[:, rows].unsqueeze(1), hs(k_, h).unsqueeze(1), hs(v_, h).unsqueeze(1))[:, 0] for h in heads])
+
+    def sampled(out):
+        return torch.stack([out[:, rows, h * D:(h + 1) * D].float() for h in heads])
+
+    out = wan_attention(q, k, v, H)
+    assert out.shape == q.shape and out.dtype == torch.bfloat16
+    ref = sampled_ref(k, v)
+    err = ((sampled(out) - ref).abs().max() / ref.abs().max()).item()
+    assert err <= 2e-2, err
+    const = wan_attention(q, k, torch.full_like(v, -1.5), H)
+    assert bool(((const.float() + 1.5).abs() <= 1.5 * 2 ** -7).all())
+    kc, vc = k[:, :512].contiguous(), v[:, :512].contiguous()
+    cross = wan_attention(q, kc, vc, H)
+    ref = sampled_ref(kc, vc)
+    err = ((sampled(cross) - ref).abs().max() / ref.abs().max()).item()
+    assert err <= 2e-2, err
+
+
 def test_full_size_attention_first_rows_match_cpu_oracle(dev):
     """A handful of query rows of one head at S = 4608 against the CPU oracle (the rest of the row space is
     covered by the invariants above)."""
