@@ -365,11 +365,42 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vw, va, acc[i][j], 0, 0, 0, 0, 0, 0);
   };
 
-  // as in fp8_gemm_kernel, with 8 MFMAs, 12 fragment reads and 4 async loads per wave and step; the
-  // fragments of step 2j + par sit in fw and fa[par]
-  auto step = [&](int j, int par) {
+  // Operands of the epilogue.  Columns >= N and rows >= M are never stored, so their addresses are clamped
+  // instead of predicated (a lane-predicated load is not batched with its neighbours).
+  EpiOperands epi;
+  float w_scale_raw = 1.0f;
+  auto load_epi = [&]() {  // loads only: whatever uses a loaded value would wait for it on the spot
+    const int n_base = n0 + wn * 128, m_base = m0 + wm * 64;
+    if (p.w_scale) w_scale_raw = *p.w_scale;
+    if (p.bias) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq)
+          epi.bias[t][rq] = *reinterpret_cast<const u32x2*>(
+              p.bias + min(n_base + t * 32 + 8 * rq + 4 * g, p.N - 4));
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) epi.bias[t][rq] = u32x2{0, 0};
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      epi.sc[t] = p.a_scale ? p.a_scale[min(m_base + t * 32 + li, p.M - 1)] : 1.0f;
+  };
+
+  // One step = 8 MFMAs per wave; the fragments of step 2j + par sit in fw and fa[par].  Between the MFMAs the
+  // wave reads the 12 fragments of the next step and issues 4 async loads of unit j + 2.  `loads` = false for
+  // the last two units (nothing is left to fetch; the odd step then waits for everything in flight);
+  // `last` = true for the very last step: no next fragments, and the registers they would occupy take the
+  // epilogue's operands instead, whose latency the remaining MFMAs cover.
+  auto step = [&](int j, int par, bool loads, bool last) {
     if (par) {
-      __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+      if (loads)
+        __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+      else
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
     } else {
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
@@ -377,12 +408,14 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
 #pragma unroll
     for (int idx = 0; idx < 8; ++idx) {
       mfma_one(par, idx);
-      if (idx & 1) {  // W tile idx/2 has been read for the last time in this step
+      if (last) {
+        if (idx == 0) load_epi();
+      } else if (idx & 1) {  // W tile idx/2 has been read for the last time in this step
         read_w(j + par, par ^ 1, idx >> 1, 0);
         read_w(j + par, par ^ 1, idx >> 1, 1);
       } else {
         read_a(par ^ 1, j + par, par ^ 1, idx >> 2, (idx >> 1) & 1);
-        issue_load(j + 2, par, idx >> 1);
+        if (loads) issue_load(j + 2, par, idx >> 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -405,29 +438,19 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
     read_a(0, 0, 0, t, 1);
   }
 
-  for (int j = 0; j < nu; ++j) {
-    step(j, 0);
-    step(j, 1);
+  for (int j = 0; j < nu - 2; ++j) {
+    step(j, 0, true, false);
+    step(j, 1, true, false);
   }
-  __builtin_amdgcn_s_waitcnt(0);  // drain the trailing async loads before the stage memory is reused
-
-  EpiOperands epi;
-  {
-    const float ws = p.w_scale ? *p.w_scale : 1.0f;
-    const int n_base = n0 + wn * 128, m_base = m0 + wm * 64;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int n = n_base + t * 32 + 8 * rq + 4 * g;
-        epi.bias[t][rq] = (p.bias && n < p.N) ? *reinterpret_cast<const u32x2*>(p.bias + n) : u32x2{0, 0};
-      }
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int m = m_base + t * 32 + li;
-      epi.sc[t] = (p.a_scale && m < p.M ? p.a_scale[m] : 1.0f) * ws;
-    }
+  if (nu >= 2) {
+    step(nu - 2, 0, false, false);
+    step(nu - 2, 1, false, false);
   }
+  step(nu - 1, 0, false, false);
+  step(nu - 1, 1, false, true);
+  __builtin_amdgcn_s_waitcnt(0);  // (the prologue's second unit, when K is a single unit)
+  epi.sc[0] *= w_scale_raw;
+  epi.sc[1] *= w_scale_raw;
   __syncthreads();  // every wave is done reading the operand stages
   store_ct_lds<RESID>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 64, lane);
 }
