@@ -195,8 +195,9 @@ template <bool RESID>
 __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][2], const EpiOperands& e,
                                               uint8_t* wave_lds, int n_base, int m_base, int lane) {
   const int g = lane >> 5, li = lane & 31;
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm) {
+  // One half (32 token rows = one accumulator column tm) at a time: scale, add bias, round, stage in LDS.  The
+  // global stores of the first half are then in flight while the second half is converted.
+  auto stage_half = [&](int tm) {
     const float sc = e.sc[tm];
     uint8_t* lrow = wave_lds + (tm * 32 + li) * kEpiPitch;
 #pragma unroll
@@ -213,9 +214,9 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
         *reinterpret_cast<u32x2*>(lrow + nl * 2) = o;
       }
     }
-  }
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the region is private to this wave
-  __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the region is private to this wave
+    __builtin_amdgcn_wave_barrier();
+  };
   const int ch = lane & 15, r0 = lane >> 4;
   const int n = n_base + ch * 8;
   const bool col_ok = n < p.N;
@@ -260,12 +261,13 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
     }
   };
   const bool interior = m_base + 64 <= p.M && n_base + 128 <= p.N;  // wave-uniform
-  if (interior) {
 #pragma unroll
-    for (int it0 = 0; it0 < 16; it0 += 8) rows8(it0, false);
-  } else {
-#pragma unroll
-    for (int it0 = 0; it0 < 16; it0 += 8) rows8(it0, true);
+  for (int tm = 0; tm < 2; ++tm) {
+    stage_half(tm);
+    if (interior)
+      rows8(tm * 8, false);
+    else
+      rows8(tm * 8, true);
   }
 }
 
