@@ -274,11 +274,16 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
 template <bool RESID>
 __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  // Both problems' arguments are fetched together with the tile counts, in one round of scalar loads, and the
+  // selected set is pinned in front of the early exit: left alone, the compiler sinks the argument loads below
+  // the exit branch, behind the wait for the counts, and every workgroup starts with two dependent round trips.
   int L = logical_tile(blockIdx.x, q.total);
-  if (L >= q.total) return;
   const bool second = L >= q.total0;
-  if (second) L -= q.total0;
   const GemmArgs p = pick(q, second);
+  asm volatile("" ::"s"(p.a), "s"(p.w), "s"(p.lda), "s"(p.ldw), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.tiles_m),
+               "s"(p.tiles_n));
+  if (L >= q.total) return;
+  if (second) L -= q.total0;
   int tm, tn;
   tile_of(L, p.tiles_m, p.tiles_n, tm, tn);
 
