@@ -9,7 +9,8 @@
 namespace dsx {
 
 // Row reductions for TPR threads per row: TPR == 64 is one wavefront per row (four rows per
-// workgroup, no LDS, no barrier); TPR == 256 is the whole workgroup on one row.
+// workgroup, no LDS, no barrier); TPR == 128 is a pair of wavefronts per row (two rows per workgroup);
+// TPR == 256 is the whole workgroup on one row.
 template <int TPR>
 __device__ __forceinline__ float row_sum(float v, float* red) {
   v = wave_sum(v);
@@ -18,6 +19,7 @@ __device__ __forceinline__ float row_sum(float v, float* red) {
   __syncthreads();  // protect `red` against a previous reduction still being read
   if ((threadIdx.x & 63) == 0) red[w] = v;
   __syncthreads();
+  if (TPR == 128) return red[w & 2] + red[w | 1];
   return red[0] + red[1] + red[2] + red[3];
 }
 template <int TPR>
@@ -28,6 +30,7 @@ __device__ __forceinline__ float row_max(float v, float* red) {
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[w] = v;
   __syncthreads();
+  if (TPR == 128) return fmaxf(red[w & 2], red[w | 1]);
   return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 }
 
@@ -53,8 +56,9 @@ __device__ __forceinline__ u32x2 quant8(const float* v, float inv) {  // |v * in
 // Emit a row held as NCH register chunks of 8 already-bf16-rounded floats.
 template <int NCH, int TPR>
 __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint16_t* y, uint8_t* q,
-                                         float* q_scale, int64_t row, float* red) {
+                                         float* q_scale, int64_t row, float* red, bool live = true) {
   const int t = threadIdx.x % TPR;
+  if (!live) nchunk = 0;  // a row slot past the last row takes part in the reductions' barriers, stores nothing
   if (y) {
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
@@ -71,7 +75,7 @@ __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint1
     }
     amax = fmaxf(row_max<TPR>(amax, red), 1e-12f);
     const float inv = 448.0f / amax;
-    if (t == 0) q_scale[row] = amax / 448.0f;
+    if (t == 0 && live) q_scale[row] = amax / 448.0f;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
       const int c = t + i * TPR;
@@ -90,7 +94,7 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
   __shared__ float red[4];
   const int t = threadIdx.x % TPR;
   int64_t row = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
-  const bool live = row < rows;  // only possible to fail for TPR == 64 (whole wavefront idle)
+  const bool live = row < rows;  // fails for whole row slots only (TPR < 256)
   if (!live) row = rows - 1;
   const int nchunk = D >> 3;
   // Chunk slots past the end of the row are clamped onto its last chunk, so that no load sits under a
@@ -196,9 +200,9 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
 #pragma unroll
       for (int j = 0; j < 8; ++j) val[i][j] = ok[i] ? val[i][j] : 0.f;
   }
-  if (!live) return;  // wave-uniform
+  if (!live && TPR == 64) return;  // wave-uniform; wider row slots share the workgroup's barriers
   emit_row<NCH, TPR>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
-                     red);
+                     red, live);
 }
 
 // RMSNorm over the whole row followed by an optional per-head RoPE (head dim 128, pairs (2i, 2i+1)):
@@ -381,10 +385,11 @@ extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale,
       rows_per_batch, (const uint16_t*)ln_w, (const uint16_t*)ln_b, eps, (uint16_t*)y, ldy,        \
       (uint8_t*)q, ldq, q_scale, rows, (int)D)
   // One wavefront per row while a row fits 6 chunks per lane and there are rows enough to fill the chip.
-  // Wider rows go to a workgroup per row: 12 chunks per lane cost 217 registers, two waves per SIMD and
-  // 266 us for 32760 x 5120; the workgroup form takes 160 us.
+  // Wider rows: 12 chunks per lane cost 217 registers, two waves per SIMD and 266 us for 32760 x 5120; a
+  // workgroup per row takes 160-175 us, a pair of wavefronts per row (two rows per workgroup) 145-150 us.
   if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_ADALN(6, 64);
   else if (D <= 2048 * 2) DSX_LAUNCH_ADALN(2, 256);
+  else if (D <= 1024 * 5 && rows >= 2048) DSX_LAUNCH_ADALN(5, 128);
   else if (D <= 2048 * 3) DSX_LAUNCH_ADALN(3, 256);
   else DSX_LAUNCH_ADALN(8, 256);
 #undef DSX_LAUNCH_ADALN

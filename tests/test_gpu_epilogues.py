@@ -164,6 +164,27 @@ def test_adaln_wave_per_row_path_many_rows(dev):
         assert torch.equal(qs.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8).reshape(-1, D), wq.view(torch.uint8))
 
 
+def test_adaln_two_wavefronts_per_row_path(dev):
+    """Rows between 4096 and 5120 wide with at least 2048 of them go two to a workgroup (a pair of wavefronts
+    each): an odd row count leaves the last workgroup's second row slot without a row, and 4608 columns leave
+    chunk slots past the end of the row."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(14)
+    for D in (5120, 4608):
+        x = torch.randn(1, 2049, D, generator=g).bfloat16()
+        mod = torch.randn(1, 2 * D, generator=g).bfloat16()
+        sc, sh = mod.chunk(2, dim=1)
+        want = O.layer_norm_modulate(x, sc[:, None], sh[:, None], 1e-6)
+        md = mod.to(dev)
+        scd, shd = md.chunk(2, dim=1)
+        y, q, qs = ops.adaln_modulate(x.to(dev), scd, shd, want_bf16=True, want_fp8=True)
+        frac, rel = _ulp_report(y.cpu(), want)
+        assert frac < 1e-3 and rel <= 2 ** -6, (D, frac, rel)
+        wq, ws = ofp8.quantize_rowwise(y.cpu().reshape(-1, D), scaled=True)
+        assert torch.equal(qs.cpu(), ws) and torch.equal(q.cpu().view(torch.uint8).reshape(-1, D), wq.view(torch.uint8))
+
+
 def test_empty_inputs_are_accepted(dev):
     """Zero rows are a valid (empty) workload for every row kernel and for the GEMM: nothing is launched and
     an empty output comes back (the reference's torch ops accept empty batches the same way)."""
