@@ -500,6 +500,7 @@ extern "C" int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float
       (const uint16_t*)x, ldx, (const uint16_t*)w, eps, rope, rope_sb, rows_per_batch, (uint16_t*)out, ldo,   \
       rows, (int)D)
   if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_RMS(6, 64);
+  else if (D > 4096 && D <= 1024 * 5 && rows >= 2048) DSX_LAUNCH_RMS(5, 128);  // as for AdaLN
   else if (D <= 2048 * 3) DSX_LAUNCH_RMS(3, 256);
   else DSX_LAUNCH_RMS(8, 256);
 #undef DSX_LAUNCH_RMS

@@ -11,7 +11,7 @@ def _cos(a, b):
     return torch.nn.functional.cosine_similarity(a.float().flatten().cpu(), b.float().flatten().cpu(), dim=0).item()
 
 
-@pytest.mark.parametrize("S,D,heads", [(24, 256, 2), (1100, 5120, 40), (7, 1536, 12)])
+@pytest.mark.parametrize("S,D,heads", [(24, 256, 2), (1100, 5120, 40), (7, 1536, 12), (2049, 5120, 40)])
 def test_rmsnorm_rows_with_rope(dev, S, D, heads):
     """RMSNorm over the full model dim then RoPE per head == wan_rms_norm + rope_apply (wan_dit.py:54-78)."""
     from diffsynth_engine_amd import ops
