@@ -455,10 +455,12 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   }
   step(nu - 1, 0, false, false);
   step(nu - 1, 1, false, true);
-  __builtin_amdgcn_s_waitcnt(0);  // (the prologue's second unit, when K is a single unit)
+  // No barrier in front of the epilogue: the last step's own barrier came after every wave's final fragment
+  // reads (lgkmcnt(0)) and after every async load had landed (vmcnt(0)), and the last step touches neither, so
+  // the ring is dead from there on and a wave may overwrite its private staging region as soon as its own MFMAs
+  // are issued -- the two waves of a SIMD then overlap one's conversion with the other's last MFMAs.
   epi.sc[0] *= w_scale_raw;
   epi.sc[1] *= w_scale_raw;
-  __syncthreads();  // every wave is done reading the operand stages
   store_ct_lds<RESID>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 64, lane);
 }
 
