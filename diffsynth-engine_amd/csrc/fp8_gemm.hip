@@ -260,7 +260,41 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
       *reinterpret_cast<u32x4*>(out_lane + (it0 + u) * out_step) = v[u];
     }
   };
+  // interior tile with a residual: each half's eight residual rows are requested before that half is
+  // converted, so that their latency passes under the conversion instead of after the LDS read-back
+  auto rows8_prefetched = [&](int it0, u32x4 (&rv)[8]) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      v[u] = *reinterpret_cast<const u32x4*>(wave_lds + ((it0 + u) * 4 + r0) * kEpiPitch + ch * 16);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      u32x4 gu = gv;
+      if (gate_per_row)
+        gu = *reinterpret_cast<const u32x4*>(
+            p.gate + (int64_t)((m_base + (it0 + u) * 4 + r0) / p.rows_per_batch) * p.gate_sb + n);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float t0 = gated ? round_bf16(bf16_lo(gu[c]) * bf16_lo(v[u][c])) : bf16_lo(v[u][c]);
+        const float t1 = gated ? round_bf16(bf16_hi(gu[c]) * bf16_hi(v[u][c])) : bf16_hi(v[u][c]);
+        v[u][c] = pack_bf16x2(bf16_lo(rv[u][c]) + t0, bf16_hi(rv[u][c]) + t1);
+      }
+      *reinterpret_cast<u32x4*>(out_lane + (it0 + u) * out_step) = v[u];
+    }
+  };
   const bool interior = m_base + 64 <= p.M && n_base + 128 <= p.N;  // wave-uniform
+  if (RESID && interior) {
+    u32x4 rva[8], rvb[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) rva[u] = *reinterpret_cast<const u32x4*>(res_lane + u * res_step);
+    stage_half(0);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) rvb[u] = *reinterpret_cast<const u32x4*>(res_lane + (8 + u) * res_step);
+    rows8_prefetched(0, rva);
+    stage_half(1);
+    rows8_prefetched(8, rvb);
+    return;
+  }
 #pragma unroll
   for (int tm = 0; tm < 2; ++tm) {
     stage_half(tm);
