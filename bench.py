@@ -291,15 +291,14 @@ def micro_benchmarks(torch, ops, dev):
         cols.append(torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1))
     rope = torch.cat(cols, dim=-2).float().contiguous()
     w1 = torch.ones(HEAD_DIM, dtype=torch.bfloat16, device=dev)
-    # q/k RMSNorm + 3-axis RoPE requested from the attention entry point: applied once into caller scratch
-    # by a row kernel ahead of the attention kernel (one C call), or inside the attention kernel's tile loads
+    # q/k RMSNorm + 3-axis RoPE requested from the attention entry point (one C call): q is treated as the
+    # attention kernel loads it, k once into caller scratch by a row kernel ahead of it.
     # "..._score_bound": the caller also states the bound on |scale * q.k| that unit RMSNorm weights imply
     # (sqrt(128), with 2 % for the bf16 roundings), which lets the kernel drop its running maximum
-    for key, in_kernel, bound in (("rmsnorm_rope_then_attention_one_call", False, 0.0),
-                                  ("rmsnorm_rope_then_attention_one_call_score_bound", False, 1.02 * HEAD_DIM ** 0.5),
-                                  ("rmsnorm_rope_in_kernel", True, 0.0)):
+    for key, bound in (("rmsnorm_rope_then_attention_one_call", 0.0),
+                       ("rmsnorm_rope_then_attention_one_call_score_bound", 1.02 * HEAD_DIM ** 0.5)):
         t = time_kernel(torch, lambda: ops.attention_bhsd(q, k, v, out=out, rope=rope, q_norm_w=w1, k_norm_w=w1,
-                                                          in_kernel=in_kernel, score_bound=bound))
+                                                          score_bound=bound))
         att[key] = {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
                     "frac_bf16_peak": round(fl / t / PEAK_BF16, 4)}
     detail["attention_S4608_H24_D128"] = att

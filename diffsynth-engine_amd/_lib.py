@@ -20,7 +20,8 @@ DSX_EALIGN = -2
 DSX_EARCH = -3
 DSX_ELAUNCH = -4
 DSX_ENULL = -5
-ABI_VERSION = 2
+DSX_EWORKSPACE = -6
+ABI_VERSION = 3
 
 
 class AttnParams(ctypes.Structure):
@@ -41,6 +42,7 @@ class AttnParams(ctypes.Structure):
         ("softmax_scale", c_float),
         ("rope", c_void_p),
         ("rope_sb", c_int64),
+        ("rope_rows", c_int64),
         ("q_norm_w", c_void_p * 2),
         ("k_norm_w", c_void_p * 2),
         ("norm_eps", c_float),

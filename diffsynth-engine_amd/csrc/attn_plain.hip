@@ -603,15 +603,19 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   return (int64_t)tail * sp.max_parts * kSlotFloats * (int64_t)sizeof(float);
 }
 
+// Compute units of the current device (0 when it cannot be asked).
 static int device_cus() {
-  static int cus = -1;
-  if (cus < 0) {
-    int dev = 0;
+  static PerDeviceOnce once;
+  static int cus[kMaxDevices];
+  int dev = -1;
+  const int rc = per_device_once(once, [&](int d) {
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
-    cus = prop.multiProcessorCount;
-  }
-  return cus;
+    if (hipGetDeviceProperties(&prop, d) != hipSuccess) return (int)DSX_EARCH;
+    cus[d] = prop.multiProcessorCount;
+    return (int)DSX_OK;
+  });
+  if (rc != DSX_OK || hipGetDevice(&dev) != hipSuccess) return 0;
+  return cus[dev];
 }
 
 int64_t attn_plain_workspace_bytes(const dsx_attn_params& p) {
@@ -621,17 +625,18 @@ int64_t attn_plain_workspace_bytes(const dsx_attn_params& p) {
 
 // `scratch` / `scratch_bytes`: optional device memory for the key-range split (may be null).
 int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_bytes, hipStream_t st) {
-  static bool attr_set = false;
-  if (!attr_set) {
+  static PerDeviceOnce attr_once;
+  const int attr_rc = per_device_once(attr_once, [](int) {
     const void* kernels[6] = {
         (const void*)attn_plain_kernel<true, true, false>,   (const void*)attn_plain_kernel<false, true, false>,
         (const void*)attn_plain_kernel<true, false, false>,  (const void*)attn_plain_kernel<false, false, false>,
         (const void*)attn_plain_kernel<true, false, true>,   (const void*)attn_plain_kernel<false, false, true>};
     for (const void* kfn : kernels)
       if (hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
-        return DSX_ELAUNCH;
-    attr_set = true;
-  }
+        return (int)DSX_ELAUNCH;
+    return (int)DSX_OK;
+  });
+  if (attr_rc != DSX_OK) return attr_rc;
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
   if (units > (1ll << 30)) return DSX_EBADSHAPE;

@@ -13,6 +13,7 @@ extern "C" const char* dsx_strerror(int code) {
     case DSX_EARCH: return "current device is not gfx950 (MI355X)";
     case DSX_ELAUNCH: return "kernel launch failed";
     case DSX_ENULL: return "required pointer is NULL";
+    case DSX_EWORKSPACE: return "scratch memory missing or too small for this call";
     default: return "unknown dsx error code";
   }
 }

@@ -4,9 +4,29 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/dsx.h"
 
 namespace dsx {
+
+// Host-side set-up that has to happen once on every device the library is used on (kernel attributes, device
+// properties): `init` runs with that device current, under a lock, until it has succeeded once.
+constexpr int kMaxDevices = 64;
+struct PerDeviceOnce {
+  std::mutex lock;
+  bool done[kMaxDevices] = {};
+};
+template <class F>
+inline int per_device_once(PerDeviceOnce& once, F&& init) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return DSX_EARCH;
+  std::lock_guard<std::mutex> guard(once.lock);
+  if (once.done[dev]) return DSX_OK;
+  const int rc = init(dev);
+  if (rc == DSX_OK) once.done[dev] = true;
+  return rc;
+}
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));

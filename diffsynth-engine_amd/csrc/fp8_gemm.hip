@@ -654,18 +654,17 @@ static int launch_gemv(const GemmArgs& p, hipStream_t st) {
 
 static int gemm_set_attributes() {
   using namespace dsx;
-  static bool attr_set = false;
-  if (!attr_set) {
+  static PerDeviceOnce once;
+  return per_device_once(once, [](int) {
     if (hipFuncSetAttribute((const void*)fp8_gemm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             kMainLdsBytes) != hipSuccess ||
         hipFuncSetAttribute((const void*)fp8_gemm_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             kMainLdsBytes) != hipSuccess ||
         hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
-      return DSX_ELAUNCH;
-    attr_set = true;
-  }
-  return DSX_OK;
+      return (int)DSX_ELAUNCH;
+    return (int)DSX_OK;
+  });
 }
 
 // Fills the tile counts and says whether the problem can run on the main 256x256 kernel.
@@ -722,6 +721,9 @@ static int gemm_fill(dsx::GemmArgs& p, const void* a, int64_t lda, const void* w
   if (!a || !w || !out) return DSX_ENULL;
   if (M < 0 || N <= 0 || K <= 0 || (K & 15) || lda < K || ldw < K || ldo < N) return DSX_EBADSHAPE;
   if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return DSX_EBADSHAPE;
+  // The kernels form per-lane operand offsets row * ld (row < 256) in 32 bits and count tiles in an int.
+  if (lda >= (1 << 24) || ldw >= (1 << 24)) return DSX_EBADSHAPE;
+  if (((M + 63) / 64) * ((N + 63) / 64) > (1ll << 30)) return DSX_EBADSHAPE;
   if ((lda & 15) || (ldw & 15) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)out & 1) ||
       ((uintptr_t)bias & 1))
     return DSX_EALIGN;

@@ -24,22 +24,22 @@ import torch
 
 from . import ops
 
-HIDDEN = 3072
-HEADS = 24
-HEAD_DIM = 128
+HEAD_DIM = 128  # the attention kernel's head width; hidden size and head count come from the checkpoint
 AXES_DIM = (16, 56, 56)
 THETA = 10000
 EPS = 1e-6
+SCALE_SUFFIX = ".weight_scale"  # per-tensor scale of an already quantised weight, as enable_fp8_linear's buffer names it
 
 
 class _Linear:
     """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias, plus optional unfused LoRA pairs."""
 
-    __slots__ = ("w", "s", "b", "n", "k", "loras", "scaled")
+    __slots__ = ("w", "s", "b", "n", "k", "loras", "scaled", "prequantised")
 
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], scaled: bool):
-        if weight.dtype == ops.FP8:
-            self.w, self.s = weight, getattr(weight, "_dsx_scale", None)
+        self.prequantised = weight.dtype == ops.FP8
+        if self.prequantised:
+            self.w, self.s = weight, None  # the scale arrives under its own key (ingest_state_dict)
         else:
             self.w, self.s = ops.quantize_weight_fp8(weight, scaled=scaled)
         self.b = None if bias is None else bias.to(torch.bfloat16).contiguous()
@@ -93,30 +93,77 @@ def _gemm_pair(la: "_Linear", pa: dict, lb: "_Linear", pb: dict):
     return ops.fp8_gemm_grouped([la.problem(**pa), lb.problem(**pb)])
 
 
+def ingest_state_dict(state_dict, device, scaled: bool, as_linear=None):
+    """Turns a checkpoint into runner storage, whatever order its keys come in (a safetensors file lists
+    ``x.bias`` before ``x.weight``; the reference loads through ``load_state_dict``, which does not care).
+
+    ``state_dict`` is a mapping or any iterable of (name, tensor) pairs; the latter lets a caller stream a
+    12B-parameter model through without ever holding it unquantised: every 2-D ``.weight`` is quantised as it
+    arrives, biases and ``.weight_scale`` entries wait until all weights are in.  ``as_linear(key, tensor)``
+    may return a 2-D view for keys that are Linear layers in disguise (a Conv3d whose kernel equals its
+    stride).  Returns (linears by name, every other tensor by full key, bf16 on the device).  A float8 weight
+    must bring its scale (``<name>.weight_scale``, which enable_fp8_linear's modules emit) when ``scaled`` is set:
+    taking it at unit scale would be wrong by 448/absmax per layer without any error."""
+    device = torch.device(device)
+    lin: Dict[str, _Linear] = {}
+    other: Dict[str, torch.Tensor] = {}
+    biases: Dict[str, torch.Tensor] = {}
+    scales: Dict[str, torch.Tensor] = {}
+    items = state_dict.items() if hasattr(state_dict, "items") else state_dict
+    for key, t in items:
+        if key.endswith(SCALE_SUFFIX):
+            scales[key[: -len(SCALE_SUFFIX)]] = t.to(device, torch.float32).reshape(())
+            continue
+        w2 = as_linear(key, t) if as_linear is not None else None
+        if w2 is None and key.endswith(".weight") and t.dim() == 2:
+            w2 = t
+        if w2 is not None:
+            lin[key[: -len(".weight")]] = _Linear(w2.to(device), None, scaled)
+        elif key.endswith(".bias"):
+            biases[key[: -len(".bias")]] = t.to(device, torch.bfloat16).contiguous()
+        else:
+            other[key] = t.to(device, torch.bfloat16).contiguous()
+    for name, sc in scales.items():
+        if name not in lin:
+            raise KeyError("%s%s has no matching weight" % (name, SCALE_SUFFIX))
+        if not lin[name].prequantised:
+            raise ValueError("%s%s given for a weight that is not float8_e4m3fn" % (name, SCALE_SUFFIX))
+        lin[name].s = sc
+    for name, b in biases.items():
+        if name in lin:
+            lin[name].b = b
+        else:
+            other[name + ".bias"] = b  # the affine bias of a norm layer
+    if scaled:
+        missing = [n for n, L in lin.items() if L.prequantised and L.s is None]
+        if missing:
+            raise ValueError("float8 weights without a scale in scaled mode (pass `<name>%s` or use scaled=False "
+                             "for reference-style unit scales): %s" % (SCALE_SUFFIX, ", ".join(missing[:4])))
+    return lin, other
+
+
 class FluxDiTRunner:
-    """Holds quantised weights of a Flux.1-dev-architecture DiT and runs one denoising step."""
+    """Holds quantised weights of a Flux-architecture DiT and runs one denoising step.  The hidden size comes
+    from the checkpoint (``x_embedder.weight``); heads are 128 wide (``heads`` = hidden / 128 unless given)."""
 
     def __init__(self, state_dict, num_double: int = 19, num_single: int = 38, scaled: bool = True,
-                 device="cuda:0", fuse_rope_in_attention: bool = False):
+                 device="cuda:0", heads: Optional[int] = None, axes_dim=AXES_DIM):
         self.device = torch.device(device)
         self.scaled = scaled
-        # q/k RMSNorm and RoPE are requested from the attention entry point.  False (default): the library
-        # gets scratch, treats k once in a row pass and q as the attention kernel loads it; True: no scratch,
-        # everything inside the attention kernel's tile loads (every query block repeats the work on k)
-        self.fuse_rope_in_attention = fuse_rope_in_attention
         self.num_double, self.num_single = num_double, num_single
-        self.lin: Dict[str, _Linear] = {}
+        self.lin, other = ingest_state_dict(state_dict, self.device, scaled)
         self.norm_w: Dict[str, torch.Tensor] = {}
-        # `state_dict` may be a mapping or any iterable of (name, tensor) pairs; the latter lets a caller
-        # stream a 12B-parameter model through without ever holding it unquantised
-        items = state_dict.items() if hasattr(state_dict, "items") else state_dict
-        for key, t in items:
-            if key.endswith(".weight") and t.dim() == 2:
-                self.lin[key[: -len(".weight")]] = _Linear(t.to(self.device), None, scaled)
-            elif key.endswith(".weight") and t.dim() == 1:
-                self.norm_w[key[: -len(".weight")]] = t.to(self.device, torch.bfloat16).contiguous()
-            elif key.endswith(".bias"):
-                self.lin[key[: -len(".bias")]].b = t.to(self.device, torch.bfloat16).contiguous()
+        for key, t in other.items():
+            if key.endswith(".weight") and t.dim() == 1:
+                self.norm_w[key[: -len(".weight")]] = t
+            else:
+                raise KeyError("unexpected entry %s %s in a Flux DiT state dict" % (key, tuple(t.shape)))
+        self.hidden = self.lin["x_embedder"].n
+        self.heads = heads if heads is not None else self.hidden // HEAD_DIM
+        self.axes_dim = tuple(axes_dim)
+        if self.heads * HEAD_DIM != self.hidden or sum(self.axes_dim) != HEAD_DIM:
+            raise ValueError("FluxDiTRunner needs hidden = heads * 128 and RoPE axes that sum to 128, got hidden %d, "
+                             "heads %d, axes %s" % (self.hidden, self.heads, self.axes_dim))
         self.has_guidance = "guidance_embedder.timestep_embedder.0" in self.lin
         # After RMSNorm over the head dim every q and k row has norm <= sqrt(128) * max|weight| and RoPE keeps
         # norms, so |q.k| / sqrt(128) <= sqrt(128) * max|w_q| * max|w_k|: the attention kernel is told so and
@@ -135,7 +182,7 @@ class FluxDiTRunner:
         self._stack_modulation()
 
     def _stack_modulation(self):
-        """One (N_total, 3072) e4m3 matrix holding every AdaLN projection, with a weight scale per row."""
+        """One (N_total, hidden) e4m3 matrix holding every AdaLN projection, with a weight scale per row."""
         names = []
         for i in range(self.num_double):
             names += [f"blocks.{i}.norm1_a.linear", f"blocks.{i}.norm1_b.linear"]
@@ -181,7 +228,7 @@ class FluxDiTRunner:
         """(B,S,64,2) fp32 (cos, sin) table of RoPEEmbedding (transformer_helper.py:39-64), float64 angles."""
         ids = torch.cat((text_ids, image_ids), dim=1).to(torch.float64)
         cols = []
-        for a, dim in enumerate(AXES_DIM):
+        for a, dim in enumerate(self.axes_dim):
             omega = 1.0 / (THETA ** (torch.arange(0, dim, 2, dtype=torch.float64, device=ids.device) / dim))
             ang = ids[..., a].unsqueeze(-1) * omega
             cols.append(torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1))
@@ -210,6 +257,7 @@ class FluxDiTRunner:
         gate_mlp (transformer_helper.py:20)."""
         pre = f"blocks.{i}."
         B, Si, d = img.shape
+        HEADS = self.heads
         St = txt.shape[1]
         ma, mb = mod_a.chunk(6, dim=1), mod_b.chunk(6, dim=1)
         L = self.lin
@@ -237,7 +285,7 @@ class FluxDiTRunner:
                            q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
                            q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
                            out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2),
-                           in_kernel=self.fuse_rope_in_attention, score_bound=self.score_bound.get(pre, 0.0))
+                           score_bound=self.score_bound.get(pre, 0.0))
         # The two streams run the same sequence on different weights (flux_dit.py:226-234): out-projection +
         # gated residual, LN-modulate, MLP + gated residual.  Each pair of linears goes out as one grouped
         # submission so that the 512-token text problem runs beside the image problem instead of after it.
@@ -273,6 +321,7 @@ class FluxDiTRunner:
         """x (B,S,d); mod (B,3d) = shift, scale, gate (transformer_helper.py:34)."""
         pre = f"single_blocks.{i}."
         B, S, d = x.shape
+        HEADS = self.heads
         L = self.lin
         shift, scale, gate = mod.chunk(3, dim=1)
         q, sc = self._modulate_q(x, scale, shift)
@@ -282,8 +331,7 @@ class FluxDiTRunner:
         nw = self.norm_w
         q_, k_, v_ = qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:]
         ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
-                           eps=EPS, out=att.transpose(1, 2), in_kernel=self.fuse_rope_in_attention,
-                           score_bound=self.score_bound.get(pre, 0.0))
+                           eps=EPS, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
         # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
         # parts and emits the e4m3 operand of proj_out with its per-token scale
         if self.scaled:
@@ -326,7 +374,7 @@ class FluxDiTRunner:
         x = x[:, St:]
         scale, shift = mods["final_norm_out.linear"].chunk(2, dim=1)  # AdaLayerNormContinuous: scale first (:333)
         q, s = self._modulate_q(x, scale, shift)
-        out = self.lin["final_proj_out"](q.view(-1, HIDDEN), s).view(B, Hh // 2, Ww // 2, C, 2, 2)
+        out = self.lin["final_proj_out"](q.view(-1, self.hidden), s).view(B, Hh // 2, Ww // 2, C, 2, 2)
         return out.permute(0, 3, 1, 4, 2, 5).reshape(B, C, Hh, Ww)
 
     __call__ = forward

@@ -8,10 +8,14 @@ that replaces ``torch.nn.functional.linear`` for its duration (fp8_linear.py:20-
 Two quantisation modes, chosen per weight:
   * reference-exact: the weight carries no scale; activation and weight are bare casts and both
     GEMM scales are 1.0 (what fp8_linear.py:35-48 computes);
-  * scaled (default of ``enable_fp8_linear`` here): the weight tensor carries ``_dsx_scale``
+  * scaled (default of ``enable_fp8_linear`` here): the Linear module gets a buffer ``weight_scale``
     (absmax/448, 0-dim fp32) and activations get a dynamic per-token scale.
-``F.linear(input, weight, bias)`` has no slot for a scale, hence the attribute on the weight.
+``F.linear(input, weight, bias)`` has no slot for a scale, so the weight Parameter carries a weak
+reference to its module (``_dsx_owner``) and the patched linear reads the buffer through it.  The buffer
+is module state: it follows ``.to()``, is written by ``state_dict()`` as ``<name>.weight_scale`` (the key
+the block runners look for) and is restored in place by ``load_state_dict``.
 """
+import weakref
 from contextlib import contextmanager
 
 import torch
@@ -20,7 +24,8 @@ import torch.nn.functional as F
 
 from . import ops
 
-SCALE_ATTR = "_dsx_scale"
+SCALE_BUFFER = "weight_scale"
+OWNER_ATTR = "_dsx_owner"
 
 
 def enable_fp8_linear(module: nn.Module, scaled: bool = True):
@@ -35,15 +40,28 @@ def _enable_fp8_linear(module: nn.Module, scaled: bool = True):
         q, scale = ops.quantize_weight_fp8(module.weight.data, scaled=scaled)
         module.weight.data = q
         if scale is not None:
-            setattr(module.weight, SCALE_ATTR, scale)
+            module.register_buffer(SCALE_BUFFER, scale)
+            setattr(module.weight, OWNER_ATTR, weakref.ref(module))
     for submodule in module.children():
         _enable_fp8_linear(submodule, scaled)
+
+
+def weight_scale_of(weight: torch.Tensor):
+    """The per-tensor scale that belongs to ``weight`` (None: a reference-style weight with unit scale)."""
+    owner = getattr(weight, OWNER_ATTR, None)
+    module = owner() if owner is not None else None
+    if module is None:
+        return None
+    scale = getattr(module, SCALE_BUFFER, None)
+    if scale is not None and scale.device != weight.device:
+        raise RuntimeError("weight_scale of a Linear is on %s, its weight on %s" % (scale.device, weight.device))
+    return scale
 
 
 def fp8_linear(input: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
     """The replacement of ``F.linear`` while ``fp8_inference`` is active."""
     origin_dtype = input.dtype
-    w_scale = getattr(weight, SCALE_ATTR, None)
+    w_scale = weight_scale_of(weight)
     if weight.dtype != ops.FP8:
         # a weight that enable_fp8_linear has not converted: cast on the fly like fp8_linear.py:36
         weight, _ = ops.quantize_weight_fp8(weight, scaled=False)

@@ -192,17 +192,17 @@ def rope_table_from_freqs(freqs: torch.Tensor) -> torch.Tensor:
 def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float] = None,
                    rope: Optional[torch.Tensor] = None, q_norm_w=None, k_norm_w=None, q2_norm_w=None,
                    k2_norm_w=None, eps: float = 1e-6, out: Optional[torch.Tensor] = None,
-                   out2: Optional[torch.Tensor] = None, in_kernel: bool = False, score_bound: float = 0.0):
+                   out2: Optional[torch.Tensor] = None, score_bound: float = 0.0, split_keys: bool = True):
     """softmax(q k^T * scale) v over the concatenation [segment 1, segment 2] of rows.
 
     q, k, v: (B,H,S,128) bf16 views with unit stride in the last dim (any other strides).
     q2/k2/v2: optional second segment (same strides as the first), appended after the first.
     rope: optional (B or 1, Sq, 64, 2) fp32 (cos, sin) table applied in-kernel to q and k;
     *_norm_w: optional (128,) bf16 RMSNorm weights applied before RoPE.
-    in_kernel: offer the library no scratch buffer.  RoPE / RMSNorm are then applied inside the attention kernel
-    as tiles are loaded (every query block repeats the work on K) and the key range of a sparsely filled last
-    round of workgroups is not split.  Default: a scratch buffer of dsx_attn_workspace_bytes is allocated here;
-    k is normalised / rotated once into it and q as the attention kernel loads it.
+    A scratch buffer of dsx_attn_workspace_bytes is allocated here when the call needs one: k is normalised /
+    rotated once into it by a row kernel (q is treated as the attention kernel loads it), and the key range of a
+    sparsely filled last round of workgroups is split over the idle compute units (split_keys=False: no scratch
+    is offered for that, one workgroup walks the whole key axis of its unit).
     score_bound: optional promise |scale * q.k| <= score_bound for every pair (after RMSNorm/RoPE); when it is
     small enough the kernel skips the running softmax maximum (same result).  0 = no promise.
     Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).
@@ -244,6 +244,7 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
         keep.append(rope)
         P.rope = _ptr(rope)
         P.rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
+        P.rope_rows = rope.shape[1]
     for i, (qw, kw) in enumerate(((q_norm_w, k_norm_w), (q2_norm_w, k2_norm_w))):
         for name, w in (("q_norm_w", qw), ("k_norm_w", kw)):
             if w is not None:
@@ -253,13 +254,13 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     P.norm_eps = eps
     P.score_bound = float(score_bound)
     lib = _lib.load()
-    if not in_kernel:
-        # scratch for the one-off q/k pre-pass and for splitting the key range of a partly filled last round
-        need = lib.dsx_attn_workspace_bytes(P)
-        if need > 0:
-            ws = torch.empty(need, dtype=torch.uint8, device=q.device)
-            keep.append(ws)
-            P.workspace, P.workspace_bytes = _ptr(ws), need
+    # scratch for the one-off k pre-pass and for splitting the key range of a partly filled last round
+    k_side = rope is not None or any(w is not None for w in (k_norm_w, k2_norm_w))
+    need = lib.dsx_attn_workspace_bytes(P) if (split_keys or k_side) else 0
+    if need > 0:
+        ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        keep.append(ws)
+        P.workspace, P.workspace_bytes = _ptr(ws), need
     rc = lib.dsx_attn_fwd(P, _stream())
     _lib.check(rc, "dsx_attn_fwd")
     return (out, out2) if q2 is not None else out

@@ -18,7 +18,7 @@ from typing import Dict
 import torch
 
 from . import ops
-from .flux_dit import _Linear
+from .flux_dit import _Linear, ingest_state_dict
 
 
 class WanDiTRunner:
@@ -26,19 +26,14 @@ class WanDiTRunner:
         self.cfg = cfg
         self.device = torch.device(device)
         self.scaled = scaled
-        self.lin: Dict[str, _Linear] = {}
-        self.vec: Dict[str, torch.Tensor] = {}
         d = cfg["dim"]
-        items = state_dict.items() if hasattr(state_dict, "items") else state_dict
-        for key, t in items:
-            if key == "patch_embedding.weight":  # Conv3d with kernel == stride == a Linear over each patch
-                self.lin["patch_embedding"] = _Linear(t.to(self.device).reshape(d, -1), None, scaled)
-            elif key.endswith(".weight") and t.dim() == 2:
-                self.lin[key[: -len(".weight")]] = _Linear(t.to(self.device), None, scaled)
-            elif key.endswith(".bias") and key[: -len(".bias")] in self.lin:
-                self.lin[key[: -len(".bias")]].b = t.to(self.device, torch.bfloat16).contiguous()
-            else:
-                self.vec[key] = t.to(self.device, torch.bfloat16).contiguous()
+
+        def conv_as_linear(key, t):  # Conv3d with kernel == stride is a Linear over each patch
+            return t.reshape(d, -1) if key == "patch_embedding.weight" else None
+
+        # key order does not matter: biases are attached once every weight is known; what is not a Linear
+        # (modulation vectors, norm weights and the affine bias of norm3) lands in `vec` under its full key
+        self.lin, self.vec = ingest_state_dict(state_dict, self.device, scaled, as_linear=conv_as_linear)
 
     # ------------------------------------------------------------------ helpers
     def _linear_bf16(self, x, name):

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define DSX_ABI_VERSION 2
+#define DSX_ABI_VERSION 3
 
 enum {
   DSX_OK = 0,
@@ -32,7 +32,8 @@ enum {
   DSX_EALIGN = -2,    /* a pointer or leading dimension not 16-byte aligned */
   DSX_EARCH = -3,     /* current device is not gfx950                       */
   DSX_ELAUNCH = -4,   /* hipLaunchKernel reported an error                  */
-  DSX_ENULL = -5      /* a required pointer is NULL                         */
+  DSX_ENULL = -5,     /* a required pointer is NULL                         */
+  DSX_EWORKSPACE = -6 /* the call needs scratch memory that was not given (or more of it) */
 };
 
 /* Version of this ABI (DSX_ABI_VERSION of the library that was built). */
@@ -81,7 +82,8 @@ int dsx_cast_fp8_scaled(const void* x, int is_fp32, const float* absmax, float* 
  * diffsynth_engine/utils/fp8_linear.py:41-48,52-59.
  *   a: (M,K) e4m3 row-major (lda); w: (N,K) e4m3 row-major (ldw), i.e. nn.Linear.weight as stored;
  *   a_scale: M fp32 or NULL (= 1); w_scale: device fp32 scalar or NULL (= 1); bias: N bf16 or NULL;
- *   out: (M,N) bf16 (ldo).  K % 16 == 0, lda/ldw % 16 == 0, ldo % 8 == 0 when N % 8 == 0.
+ *   out: (M,N) bf16 (ldo).  K % 16 == 0, lda/ldw % 16 == 0, ldo % 8 == 0 when N % 8 == 0;
+ *   M, N, K <= 2^30, lda and ldw < 2^24 (operand offsets inside a tile are 32-bit), ceil(M/64)*ceil(N/64) <= 2^30.
  */
 int dsx_fp8_gemm(const void* a, int64_t lda, const void* w, int64_t ldw, const float* a_scale,
                  const float* w_scale, const void* bias, void* out, int64_t ldo, int64_t M,
@@ -163,10 +165,13 @@ typedef struct dsx_attn_params {
   /* Optional fused pre-processing of q and k (NULL = off):
    *   rope      : fp32 table (rope_sb*b + pos*128 + 2*i + {0,1}) = (cos, sin) of pair i at
    *               joint position pos (segment 0 rows first); applied to q and k on pairs (2i,2i+1),
-   *               result rounded to bf16.
+   *               result rounded to bf16.  The table holds rope_rows rows per batch entry; rope_rows must
+   *               be at least sq[0]+sq[1] (= skv[0]+skv[1]: the option is for self / joint attention), and
+   *               rope_sb is 0 (one table for every batch entry) or at least rope_rows*128.
    *   q_norm_w/k_norm_w[g] : bf16 (128,) RMSNorm weight of segment g; y = bf16(bf16(x*rsqrt(ms+eps))*w). */
   const float* rope;
   int64_t rope_sb;
+  int64_t rope_rows;
   const void* q_norm_w[2];
   const void* k_norm_w[2];
   float norm_eps;
@@ -176,13 +181,14 @@ typedef struct dsx_attn_params {
    * RMSNorm over head_dim with weights wq, wk: head_dim * max|wq| * max|wk| * softmax_scale.  A promise
    * that does not hold can overflow exp2. */
   float score_bound;
-  /* Optional scratch owned by the caller (NULL = none, 16-byte aligned), used for two things when it is
-   * large enough (dsx_attn_workspace_bytes gives the size that enables both):
-   *  - fused pre-processing: with 2*batch*heads*Skv*128 bytes, k is normalised/rotated ONCE into it by a
-   *    row kernel and the attention kernel reads it from there (q is treated as it is loaded, each row
-   *    once); without it the same arithmetic is applied inside the attention kernel as tiles are loaded,
-   *    where every query block repeats the work on K;
-   *  - load balance: when the (batch, head, 256-query block) units do not fill the last round of
+  /* Scratch owned by the caller (NULL = none, 16-byte aligned); dsx_attn_workspace_bytes gives the size that
+   * serves both uses:
+   *  - fused pre-processing of k (rope, k_norm_w): k is normalised/rotated ONCE into the first
+   *    2*batch*heads*Skv*128 bytes by a row kernel and the attention kernel reads it from there (every query
+   *    block of a head reads all of that head's k, so the work is not repeated per block); q is treated as the
+   *    attention kernel loads it, each row once, and needs no scratch.  A call that asks for rope or k_norm_w
+   *    without that much scratch returns DSX_EWORKSPACE;
+   *  - load balance (optional): when the (batch, head, 256-query block) units do not fill the last round of
    *    workgroups, the key ranges of that round's units are cut into equal pieces over all compute units
    *    and a second kernel merges the partial softmax results held in the scratch.
    * Calls that share a scratch must not overlap. */
@@ -192,8 +198,8 @@ typedef struct dsx_attn_params {
 
 int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
 
-/* Scratch bytes with which dsx_attn_fwd(p) uses every option described at `workspace` (0: none would be
- * used).  Reads the shapes and the fused-option pointers of *p only; launches nothing.  No counterpart in
+/* Scratch bytes with which dsx_attn_fwd(p) runs and uses every option described at `workspace` (0: none is
+ * needed or would be used).  Reads the shapes and the fused-option pointers of *p only; launches nothing.  No counterpart in
  * the reference, whose attention backends allocate their own temporaries. */
 int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p);
 

@@ -8,6 +8,13 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+def row_rel_err(got, want):
+    """Attention error norm of every GPU test: for each row of the last dim (one query of one head), the largest
+    |got - want| divided by the largest |want| of that same row; the result is the worst row."""
+    got, want = got.float(), want.float()
+    return ((got - want).abs().amax(-1) / want.abs().amax(-1).clamp_min(1e-30)).max().item()
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 

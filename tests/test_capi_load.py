@@ -32,9 +32,9 @@ def test_abi_version_and_strerror():
     from diffsynth_engine_amd import _lib
 
     lib = _lib.load()
-    assert lib.dsx_abi_version() == 2
+    assert lib.dsx_abi_version() == 3
     assert _lib.strerror(0) == "ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
     assert "unknown" in _lib.strerror(-99)
 
@@ -42,9 +42,9 @@ def test_abi_version_and_strerror():
 def test_attn_params_struct_layout_matches_header():
     from diffsynth_engine_amd import _lib
 
-    # 8 + 4 pointers/int64 pairs (12*8*... ) : q,k,v,o,sq,skv = 6*16; 12 strides*8; 3 int32 + float; rope, rope_sb;
-    # 2*16 norm pointers; float + int32; workspace pointer + byte count
-    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 32 + 8 + 16
+    # q,k,v,o,sq,skv = 6*16; 12 stride pairs * 16; 3 int32 + float; rope, rope_sb, rope_rows;
+    # 2*16 norm pointers; two floats; workspace pointer + byte count
+    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 8 + 32 + 8 + 16
 
 
 def test_null_and_shape_errors_without_touching_the_gpu():
@@ -163,3 +163,60 @@ def test_graphed_step_refuses_host_inputs():
 
     with pytest.raises(RuntimeError):
         GraphedStep(lambda **kw: None, x=torch.zeros(4))
+
+
+def _host_attn_params(buf, sq=64, skv=64):
+    """dsx_attn_params over a host buffer: good enough for everything dsx_attn_fwd checks before it launches."""
+    from diffsynth_engine_amd import _lib
+
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+    P = _lib.AttnParams()
+    for name in ("q", "k", "v", "o"):
+        getattr(P, name)[0] = p16
+        getattr(P, name + "_sb")[0], getattr(P, name + "_sh")[0], getattr(P, name + "_ss")[0] = 0, 128, 128
+    P.sq[0], P.skv[0], P.batch, P.heads, P.head_dim = sq, skv, 1, 1, 128
+    P.softmax_scale = 0.0884
+    return P, p16
+
+
+def test_attention_refuses_what_its_kernels_would_mis_address():
+    """Checked on the host before any launch: overlapping key/value rows, a RoPE table with fewer rows than the
+    joint sequence, RoPE with Sq != Skv, and k-side pre-processing without the scratch it needs."""
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(1 << 16)
+    P, p16 = _host_attn_params(buf)
+    P.k_ss[0] = 64
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE
+    P, p16 = _host_attn_params(buf)
+    P.v_ss[0] = 120
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE
+    P, p16 = _host_attn_params(buf)
+    P.rope, P.rope_rows = p16, 63  # one row short
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE
+    P.rope_rows = 64
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EWORKSPACE  # k has to be rotated into scratch that was not given
+    P.workspace, P.workspace_bytes = p16, 2 * 64 * 128 - 16
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EWORKSPACE  # too small
+    P, p16 = _host_attn_params(buf, sq=64, skv=32)
+    P.rope, P.rope_rows = p16, 64
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE  # fused RoPE is for self / joint attention
+    P, p16 = _host_attn_params(buf)
+    P.k_norm_w[0] = p16
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EWORKSPACE
+    with pytest.raises(ValueError):
+        _lib.check(_lib.DSX_EWORKSPACE, "x")
+
+
+def test_gemm_refuses_leading_dimensions_beyond_its_32_bit_tile_offsets():
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096)
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+    big = 1 << 24
+    assert lib.dsx_fp8_gemm(p16, big, p16, 128, None, None, None, p16, 256, 16, 256, 128, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_fp8_gemm(p16, 128, p16, big, None, None, None, p16, 256, 16, 256, 128, None) == _lib.DSX_EBADSHAPE
+    n = 1 << 30  # 2^24 x 2^24 tiles of 64 x 64
+    assert lib.dsx_fp8_gemm(p16, 128, p16, 128, None, None, None, p16, n, n, n, 128, None) == _lib.DSX_EBADSHAPE

@@ -56,10 +56,9 @@ def test_deeper_step_matches_oracle(dev):
     sd_dev = {k: v.to(dev) for k, v in sd.items()}
     inp_dev = {k: v.to(dev) for k, v in inp.items()}
     want_dev = oflux.flux_dit_forward(oflux.Params(sd_dev, "fp8_scaled"), **inp_dev, num_double=4, num_single=6).cpu()
-    for fuse in (False, True):
-        got = FluxDiTRunner(sd_dev, 4, 6, scaled=True, device=dev, fuse_rope_in_attention=fuse)(**inp_dev).cpu()
-        assert _cos(got, want) >= 0.99
-        assert _cos(got, want) >= _floor(want, want_dev), (fuse, _cos(got, want), _cos(want, want_dev))
+    got = FluxDiTRunner(sd_dev, 4, 6, scaled=True, device=dev)(**inp_dev).cpu()
+    assert _cos(got, want) >= 0.99
+    assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
 
 
 def test_blocks_teacher_forced_against_oracle(dev):

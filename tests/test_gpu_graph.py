@@ -19,13 +19,12 @@ def _inputs(side, n_txt, seed, dev):
                 guidance=torch.tensor([3.5], device=dev), text_ids=torch.zeros(1, n_txt, 3, device=dev))
 
 
-@pytest.mark.parametrize("fuse", [False, True])
-def test_flux_step_graph_replays_equal_eager(dev, fuse):
+def test_flux_step_graph_replays_equal_eager(dev):
     from diffsynth_engine_amd.flux_dit import FluxDiTRunner
     from diffsynth_engine_amd.graph import GraphedStep
 
     sd = {k: v.to(dev) for k, v in oflux.init_params(2, 2, dtype=torch.bfloat16, seed=11, bias_std=0.02).items()}
-    runner = FluxDiTRunner(sd, 2, 2, scaled=True, device=dev, fuse_rope_in_attention=fuse)
+    runner = FluxDiTRunner(sd, 2, 2, scaled=True, device=dev)
     step = GraphedStep(runner, **_inputs(32, 64, 0, dev))
     for r in range(1, 5):
         inp = _inputs(32, 64, r, dev)
