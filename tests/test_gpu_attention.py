@@ -225,10 +225,14 @@ def test_key_range_split_of_the_last_round(dev, H, Sq, Skv, qscale, bound):
     P.sq[0], P.skv[0], P.batch, P.heads, P.head_dim = Sq, Skv, 1, H, 128
     assert _lib.load().dsx_attn_workspace_bytes(P) > 0  # this shape does take the split path
     got = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=bound).cpu()
-    assert _rel_err(got, want) <= TOL
+    # The kernel multiplies q by scale * log2(e) once and rounds the product to bf16 (2^-9 relative), so a score s
+    # carries an absolute error of about |s| * 2^-9 in the exponent.  For N(0,1) operands (|s| of a few units) that
+    # is far inside the bar; the x12 case is there to force the softmax references of the parts apart (|s| up to
+    # ~60, near one-hot rows that flip between two values), and is held to 3 x the bar.
+    assert _rel_err(got, want) <= (TOL if qscale <= 1.0 else 3 * TOL)
     # the unsplit kernel (no scratch offered) gives the same rows up to the order of the fp32 sums
     same = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), score_bound=bound, split_keys=False).cpu()
-    assert _rel_err(got, same) <= 2 ** -7
+    assert _rel_err(got, same) <= (2 ** -7 if qscale <= 1.0 else 2 ** -6)  # (a moved reference re-rounds P once more)
 
 
 def test_key_range_split_joint_two_segments(dev):
