@@ -91,6 +91,8 @@ SIGNATURES = {
                                      c_int64, c_void_p, c_int64, c_int64, c_void_p]),
     "dsx_attn_fwd": (c_int, [ctypes.POINTER(AttnParams), c_void_p]),
     "dsx_attn_workspace_bytes": (c_int64, [ctypes.POINTER(AttnParams)]),
+    "dsx_attn_fwd_static": (c_int, [ctypes.POINTER(AttnParams), c_void_p]),
+    "dsx_attn_static_scratch_bytes": (c_int64, []),
     "dsx_rmsnorm_rope": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int64,
                                  c_int64, c_void_p, c_int64, c_int64, c_int64, ctypes.c_int32, ctypes.c_int32,
                                  c_int64, c_void_p]),

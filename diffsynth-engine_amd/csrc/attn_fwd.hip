@@ -1,10 +1,10 @@
-// Attention entry point of the C ABI (dsx_attn_fwd) and the row kernels that
+// Attention entry points of the C ABI (dsx_attn_fwd and its allocation-free twin) and the row kernels that
 // apply the per-head RMSNorm and the RoPE rotation to q and k ahead of the attention kernel.
 //
 // RMSNorm / RoPE requested from dsx_attn_fwd are applied to q inside the attention kernel (attn_plain.hip: every
 // query row is read exactly once there) and to k by ONE pass of rmsnorm_rope_kernel into scratch memory (every
 // query block of a head reads all of that head's k, so per-block recomputation would repeat the work 18 times at
-// 4608 tokens).  The scratch is the caller's.
+// 4608 tokens).  The scratch is the caller's (dsx_attn_fwd) or a static device array (dsx_attn_fwd_static).
 #include "attn_internal.h"
 #include "common.h"
 
@@ -191,6 +191,43 @@ extern "C" int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p) {
   const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
   if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 30) || Skv > (1ll << 30)) return 0;
   return attn_k_copy_bytes(p) + attn_plain_workspace_bytes(*p);
+}
+
+// ---- the allocation-free twin: the same launches over a static device array ------------------------------
+// Every GPU the library runs on holds its own copy of the array at its own address; the host-side name is only
+// a handle for hipGetSymbolAddress, never a pointer a kernel could use.
+namespace {
+__device__ __align__(256) unsigned char scratch[DSX_ATTN_STATIC_SCRATCH_BYTES];
+dsx::PerDeviceOnce g_scratch_once;
+void* g_scratch_ptr[dsx::kMaxDevices];  // per device, resolved on the first call made with that device current
+}  // namespace
+
+// Device address of the current device's copy of `scratch` (resolved once per device, under a lock).
+static int attn_static_scratch(void** out) {
+  const int rc = dsx::per_device_once(g_scratch_once, [](int dev) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return (int)DSX_ELAUNCH;
+    g_scratch_ptr[dev] = ptr;
+    return (int)DSX_OK;
+  });
+  if (rc != DSX_OK) return rc;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= dsx::kMaxDevices) return DSX_EARCH;
+  *out = g_scratch_ptr[dev];
+  return DSX_OK;
+}
+
+extern "C" int64_t dsx_attn_static_scratch_bytes(void) { return DSX_ATTN_STATIC_SCRATCH_BYTES; }
+
+extern "C" int dsx_attn_fwd_static(const dsx_attn_params* p, void* stream) {
+  int rc = attn_validate(p);
+  if (rc != DSX_OK) return rc;
+  if (p->workspace) return DSX_EBADSHAPE;  // this entry point owns its scratch; a caller's buffer goes to dsx_attn_fwd
+  const int64_t need = dsx_attn_workspace_bytes(p);
+  if (need > DSX_ATTN_STATIC_SCRATCH_BYTES) return DSX_EWORKSPACE;
+  void* ws = nullptr;
+  if (need > 0 && (rc = attn_static_scratch(&ws)) != DSX_OK) return rc;
+  return attn_run(p, ws, need > 0 ? DSX_ATTN_STATIC_SCRATCH_BYTES : 0, (hipStream_t)stream);
 }
 
 extern "C" int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss,

@@ -192,7 +192,8 @@ def rope_table_from_freqs(freqs: torch.Tensor) -> torch.Tensor:
 def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float] = None,
                    rope: Optional[torch.Tensor] = None, q_norm_w=None, k_norm_w=None, q2_norm_w=None,
                    k2_norm_w=None, eps: float = 1e-6, out: Optional[torch.Tensor] = None,
-                   out2: Optional[torch.Tensor] = None, score_bound: float = 0.0, split_keys: bool = True):
+                   out2: Optional[torch.Tensor] = None, score_bound: float = 0.0, split_keys: bool = True,
+                   static_scratch: bool = False):
     """softmax(q k^T * scale) v over the concatenation [segment 1, segment 2] of rows.
 
     q, k, v: (B,H,S,128) bf16 views with unit stride in the last dim (any other strides).
@@ -203,6 +204,9 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     rotated once into it by a row kernel (q is treated as the attention kernel loads it), and the key range of a
     sparsely filled last round of workgroups is split over the idle compute units (split_keys=False: no scratch
     is offered for that, one workgroup walks the whole key axis of its unit).
+    static_scratch: go through dsx_attn_fwd_static, the entry point that allocates nothing: the library's own
+    static device array serves as scratch (calls on one GPU must then not overlap) and a call that needs more
+    than it holds raises.
     score_bound: optional promise |scale * q.k| <= score_bound for every pair (after RMSNorm/RoPE); when it is
     small enough the kernel skips the running softmax maximum (same result).  0 = no promise.
     Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).
@@ -255,6 +259,9 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     P.score_bound = float(score_bound)
     lib = _lib.load()
     # scratch for the one-off k pre-pass and for splitting the key range of a partly filled last round
+    if static_scratch:
+        _lib.check(lib.dsx_attn_fwd_static(P, _stream()), "dsx_attn_fwd_static")
+        return (out, out2) if q2 is not None else out
     k_side = rope is not None or any(w is not None for w in (k_norm_w, k2_norm_w))
     need = lib.dsx_attn_workspace_bytes(P) if (split_keys or k_side) else 0
     if need > 0:

@@ -204,6 +204,25 @@ int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
 int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p);
 
 /*
+ * dsx_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same results, but the scratch is a
+ * static device array of DSX_ATTN_STATIC_SCRATCH_BYTES inside the library instead of `workspace`, which must be
+ * NULL.  It has no counterpart in the reference, whose attention backends allocate their temporaries themselves.
+ * Calls whose dsx_attn_workspace_bytes exceeds the array return DSX_EWORKSPACE before anything is launched; the
+ * limit (64 MiB) covers the k copy of a fused RMSNorm/RoPE call at batch * heads * Skv <= 262144 rows (Flux at
+ * 1024 x 1024: 24 heads x 4608 tokens = 27 MiB) and the partial results of a key-range split of a few dozen units.  Each GPU the library runs on holds its own copy of the array until the process
+ * ends.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (different streams, or
+ * threads) race; calls on one stream are ordered and safe.  Nothing in the array has to start at zero: every
+ * byte a call reads was written earlier in that same call.  The entry point calls no hipMalloc, hipFree or other
+ * allocating routine.
+ */
+#define DSX_ATTN_STATIC_SCRATCH_BYTES (64ll << 20)
+int dsx_attn_fwd_static(const dsx_attn_params* p, void* stream);
+
+/* DSX_ATTN_STATIC_SCRATCH_BYTES of the library that was built. */
+int64_t dsx_attn_static_scratch_bytes(void);
+
+/*
  * Standalone RMSNorm + RoPE of q and k (same arithmetic and rounding points as the fused
  * option of dsx_attn_fwd), written to a strided (B,H,S,128) bf16 view; `out` may be `x` itself
  * (in place).  One tensor per call.

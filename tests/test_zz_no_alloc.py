@@ -1,0 +1,89 @@
+"""The allocation-free attention entry point (dsx_attn_fwd_static: scratch in a static device array of the
+library) against dsx_attn_fwd with caller scratch, through the C ABI: bit-equal outputs on two calls in a row,
+the second smaller than the first, for both uses of the scratch (the k copy of a fused RMSNorm + RoPE call and
+the partial results of the key-range split)."""
+import ctypes
+
+import pytest
+import torch
+
+from oracle import dit_ops as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _params(_lib, q, k, v, o, rope=None, wq=None, wk=None):
+    B, H, Sq, D = q.shape
+    P = _lib.AttnParams()
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o)):
+        getattr(P, name)[0] = t.data_ptr()
+        getattr(P, name + "_sb")[0], getattr(P, name + "_sh")[0], getattr(P, name + "_ss")[0] = t.stride()[:3]
+    P.sq[0], P.skv[0], P.batch, P.heads, P.head_dim = Sq, k.shape[2], B, H, D
+    P.softmax_scale = D ** -0.5
+    P.norm_eps = 1e-6
+    if rope is not None:
+        P.rope, P.rope_sb, P.rope_rows = rope.data_ptr(), 0, rope.shape[1]
+    if wq is not None:
+        P.q_norm_w[0] = wq.data_ptr()
+    if wk is not None:
+        P.k_norm_w[0] = wk.data_ptr()
+    return P
+
+
+def _both(dev, H, S, fused, seed):
+    """Runs one call through each entry point on the same operands; returns (static output, workspace output, q, k, v
+    as the kernel saw them)."""
+    from diffsynth_engine_amd import _lib, ops
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(1, H, S, 128, generator=g).bfloat16().to(dev) for _ in range(3)]
+    rope = wq = wk = None
+    if fused:
+        ids = torch.zeros(1, S, 3)
+        ids[0, :, 1] = torch.arange(S) // 16
+        ids[0, :, 2] = torch.arange(S) % 16
+        rope = ops.rope_table_from_freqs(O.rope_table(ids, (16, 56, 56), 10000)).to(dev)
+        wq = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16().to(dev)
+        wk = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16().to(dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    o_static = torch.zeros(1, H, S, 128, dtype=torch.bfloat16, device=dev)
+    o_ws = torch.zeros_like(o_static)
+    P = _params(_lib, q, k, v, o_ws, rope, wq, wk)
+    need = lib.dsx_attn_workspace_bytes(P)
+    assert 0 < need <= lib.dsx_attn_static_scratch_bytes()
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    P.workspace, P.workspace_bytes = ws.data_ptr(), need
+    assert lib.dsx_attn_fwd(P, stream) == 0
+    Ps = _params(_lib, q, k, v, o_static, rope, wq, wk)
+    before = torch.cuda.memory_allocated(dev)
+    assert lib.dsx_attn_fwd_static(Ps, stream) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated(dev) == before
+    return o_static, o_ws
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_static_scratch_entry_point_equals_the_workspace_one_on_two_calls_in_a_row(dev, fused):
+    # fused: the scratch holds the normalised / rotated copy of k.  Not fused: 3 heads x 8 query blocks = 24 units
+    # on 256 compute units, which takes the key-range split (partial results in the scratch).
+    shapes = [(4, 1536), (2, 520)] if fused else [(3, 2048), (1, 2048)]
+    for i, (H, S) in enumerate(shapes):
+        o_static, o_ws = _both(dev, H, S, fused, seed=40 + i)
+        assert torch.isfinite(o_static.float()).all().item()
+        assert o_static.float().abs().max().item() > 0
+        assert torch.equal(o_static, o_ws), (fused, H, S)
+
+
+def test_static_scratch_entry_point_refuses_what_does_not_fit(dev):
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    H, S = 40, 8192  # k copy: 40 * 8192 * 256 B = 80 MiB > 64 MiB
+    q = torch.zeros(1, H, S, 128, dtype=torch.bfloat16, device=dev)
+    rope = torch.zeros(1, S, 64, 2, device=dev)
+    P = _params(_lib, q, q, q, torch.empty_like(q), rope)
+    assert lib.dsx_attn_workspace_bytes(P) > lib.dsx_attn_static_scratch_bytes()
+    assert lib.dsx_attn_fwd_static(P, None) == _lib.DSX_EWORKSPACE
+    P.workspace, P.workspace_bytes = q.data_ptr(), 16
+    assert lib.dsx_attn_fwd_static(P, None) == _lib.DSX_EBADSHAPE  # a caller's buffer belongs to dsx_attn_fwd
