@@ -129,15 +129,33 @@ def run_wan(args, torch, dev):
     x = torch.randn(1, 16, 21, 60, 104, generator=g, device=dev).to(torch.bfloat16)
     ctx = torch.randn(1, 512, 4096, generator=g, device=dev).to(torch.bfloat16)
     t = torch.tensor([500.0], device=dev)
+    from diffsynth_engine_amd import ops
+
     for _ in range(args.warmup):
         out = runner(x, ctx, t)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = runner(x, ctx, t)
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    with AttnTimer(torch, ops) as at, GemmTimer(torch, ops) as gt:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = runner(x, ctx, t)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        n_attn, attn_flops, attn_secs = at.summary()
+        n_gemm, gemm_flops, gemm_secs = gt.summary()
     assert torch.isfinite(out.float()).all().item(), "non-finite output"
+    # sampled-row parity of the timed configuration: the last layer's self-attention shape through the same entry
+    # point against torch's fp32 SDPA on a few query rows of three heads
+    gq = torch.Generator(device=dev).manual_seed(1)
+    q, k, v = [torch.randn(1, 32760, 5120, generator=gq, device=dev, dtype=torch.bfloat16) for _ in range(3)]
+    o = runner._attention(q, k, v).view(1, 32760, 40, 128)
+    rows = torch.tensor([0, 255, 16383, 32759], device=dev)
+    for h in (0, 21, 39):
+        hs = lambda tt: tt.view(1, 32760, 40, 128)[:, :, h].float()
+        ref = torch.nn.functional.scaled_dot_product_attention(hs(q)[:, rows].unsqueeze(1), hs(k).unsqueeze(1),
+                                                               hs(v).unsqueeze(1))[:, 0]
+        err = ((o[:, rows, h].float() - ref).abs().amax(-1) / ref.abs().amax(-1)).max().item()
+        assert err <= 2e-2, "attention row check failed: %g" % err
+    del q, k, v, o
     S, d, f, L = 21 * 30 * 52, cfg["dim"], cfg["ffn_dim"], cfg["num_layers"]
     gemm = L * (2.0 * S * d * d * 4 + 2.0 * S * d * f * 2 + 2.0 * S * d * d * 2 + 2.0 * 512 * d * d * 2)
     attn = L * (4.0 * S * S * d + 4.0 * S * 512 * d)
@@ -149,8 +167,18 @@ def run_wan(args, torch, dev):
         "data": "synthetic",
         "config": {"workload": "BASELINE configs[4]: Wan2.1-14B-architecture DiT, one denoising step, %d layers, "
                                "32760 video tokens (21x60x104 latent) + 512 text tokens, batch 1, random init" % L},
+        # dominant kernel: attn_plain_kernel (53 % of the step's flops); self- and cross-attention launches together
+        "roofline": {"bound": "mfma", "achieved": round(attn_flops / attn_secs / 1e12, 1), "peak": PEAK_BF16 / 1e12,
+                     "unit": "TFLOP/s", "frac": round(attn_flops / attn_secs / PEAK_BF16, 4), "traffic": None,
+                     "kernel": "attn_plain_kernel", "launches": n_attn,
+                     "avg_launch_us": round(attn_secs / max(n_attn, 1) * 1e6, 1)},
+        "detail": {"fp8_gemm_in_step": {"launches": n_gemm, "tflops": round(gemm_flops / gemm_secs / 1e12, 1),
+                                        "frac_fp8_peak": round(gemm_flops / gemm_secs / PEAK_FP8, 4),
+                                        "ms_per_step": round(gemm_secs * 1e3 / args.steps, 1)},
+                   "attention_in_step": {"ms_per_step": round(attn_secs * 1e3 / args.steps, 1)}},
         "step_roofline": {"algorithmic_tflop": round((gemm + attn) / 1e12, 1), "ideal_ms": round(t_ideal * 1e3, 1),
-                          "frac": round(t_ideal * 1e3 / ms, 4)}}))
+                          "frac": round(t_ideal * 1e3 / ms, 4)},
+        "cpu_baseline": None if args.no_cpu_baseline else wan_cpu_baseline(cfg, S)}))
 
 
 def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
@@ -211,6 +239,40 @@ class GemmTimer:
         secs = sum(e0.elapsed_time(e1) for e0, e1, _ in self.records) * 1e-3
         flops = sum(f for _, _, f in self.records)
         return len(self.records), flops, secs
+
+
+class AttnTimer:
+    """Brackets every ops.attention_bhsd call of a step with events on the launch stream and accumulates the
+    algorithmic flops 4 * Sq * Skv * D * H * B of each (a call with fused q/k pre-processing includes its k row pass)."""
+
+    def __init__(self, torch, ops):
+        self.torch, self.ops, self.records = torch, ops, []
+        self._orig = ops.attention_bhsd
+
+    def __enter__(self):
+        torch, orig, rec = self.torch, self._orig, self.records
+
+        def timed(q, k, v, *args, q2=None, k2=None, **kw):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = orig(q, k, v, *args, q2=q2, k2=k2, **kw)
+            e1.record()
+            B, H, Sq, D = q.shape
+            Sq += 0 if q2 is None else q2.shape[2]
+            Skv = k.shape[2] + (0 if k2 is None else k2.shape[2])
+            rec.append((e0, e1, 4.0 * B * H * Sq * Skv * D))
+            return out
+
+        self.ops.attention_bhsd = timed
+        return self
+
+    def __exit__(self, *exc):
+        self.ops.attention_bhsd = self._orig
+
+    def summary(self):
+        self.torch.cuda.synchronize()
+        secs = sum(e0.elapsed_time(e1) for e0, e1, _ in self.records) * 1e-3
+        return len(self.records), sum(f for _, _, f in self.records), secs
 
 
 def time_kernel(torch, fn, args_list=None, reps=10):
@@ -318,13 +380,15 @@ def micro_benchmarks(torch, ops, dev):
     t3q = time_kernel(torch, lambda h: ops.gelu_tanh(h, want_bf16=False, want_fp8=True), hs_rot)
     del hs_rot
     n = S * HIDDEN
+    def hbm(t, nbytes):  # algorithmic bytes over time, and as a fraction of the 8 TB/s peak
+        return {"us": round(t * 1e6, 1), "gbps": round(nbytes / t / 1e9, 1), "frac_hbm": round(nbytes / t / PEAK_HBM, 4)}
+
     detail["epilogues"] = {
-        "adaln_modulate_bf16": {"us": round(t1 * 1e6, 1), "gbps": round(4 * n / t1 / 1e9, 1)},
-        "adaln_modulate_fp8": {"us": round(t1q * 1e6, 1), "gbps": round(3 * n / t1q / 1e9, 1)},
-        "gated_residual": {"us": round(t2 * 1e6, 1), "gbps": round(6 * n / t2 / 1e9, 1)},
-        "gelu_tanh_bf16": {"us": round(t3 * 1e6, 1), "gbps": round(16 * n / t3 / 1e9, 1)},
-        "gelu_tanh_fp8": {"us": round(t3q * 1e6, 1), "gbps": round(12 * n / t3q / 1e9, 1)},
+        "adaln_modulate_bf16": hbm(t1, 4 * n), "adaln_modulate_fp8": hbm(t1q, 3 * n), "gated_residual": hbm(t2, 6 * n),
+        "gelu_tanh_bf16": hbm(t3, 16 * n), "gelu_tanh_fp8": hbm(t3q, 12 * n),
     }
+    for kn, v in gem.items():
+        v["quant_frac_hbm"] = round(v["quant_gbps"] * 1e9 / PEAK_HBM, 4)
     return detail
 
 
@@ -364,6 +428,92 @@ def cpu_baseline(num_double, num_single):
             "sample": "oracle fp32 on host: 1 double block (%.2f s) + 1 single block (%.2f s) at 4096+512 tokens, "
                       "mean of %d runs each, extrapolated x%d + x%d (embedders and final layer excluded)"
                       % (td, ts, reps, num_double, num_single)}
+
+
+def _median_time(fn, warm, reps):
+    for _ in range(warm):
+        fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[len(ts) // 2]
+
+
+def cpu_config_legs():
+    """The CPU torch path of BASELINE configs[0..2] on the host cores, each at its full size:
+    configs[0] the fp32 joint block at 1024 image + 256 text tokens with torch SDPA (the configuration IS this CPU
+    run; median of 5 after 3 warm-ups); configs[1] the fp32 matmul of the dequantised operands plus bias at
+    M = 4608 for the four (K, N); configs[2] fp32 SDPA of (1, 24, 4608, 128) operands (RMSNorm / RoPE are
+    negligible beside it)."""
+    import torch
+
+    from oracle import dit_ops as O
+    from oracle import flux as oflux
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    legs = {"cores": torch.get_num_threads()}
+    g = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        sd = oflux.init_params(1, 0, dtype=torch.float32, seed=0)
+        P = oflux.Params(sd, "plain")
+        img, txt, cond = torch.randn(1, 1024, HIDDEN, generator=g), torch.randn(1, 256, HIDDEN, generator=g), \
+            torch.randn(1, HIDDEN, generator=g)
+        ids = torch.cat([torch.zeros(1, 256, 3), oflux.image_ids(64, 64, 1, "cpu", torch.float32)], dim=1)
+        freqs = O.rope_table(ids, oflux.AXES_DIM, oflux.THETA)
+        sdpa = torch.nn.functional.scaled_dot_product_attention
+        t = _median_time(lambda: oflux.joint_block(P, 0, img, txt, cond, freqs, attn=sdpa), 3, 5)
+        gf = (2 * 1280 * HIDDEN * 12 * HIDDEN + 4 * 1280 * 1280 * HIDDEN) / 1e9
+        legs["config0_joint_block_1024+256_fp32"] = {"ms": round(t * 1e3, 1), "gflops": round(gf / t, 1),
+                                                     "sample": "full size, median of 5 after 3 warm-ups"}
+        del sd, P
+        mm = {}
+        for K, N in ((3072, 9216), (3072, 3072), (3072, 12288), (12288, 3072)):
+            a, w, b = torch.randn(N_IMG + N_TXT, K, generator=g), torch.randn(N, K, generator=g), torch.randn(N, generator=g)
+            t = _median_time(lambda: torch.addmm(b, a, w.t()), 1, 3)
+            mm[f"{K}x{N}"] = {"ms": round(t * 1e3, 1), "gflops": round(2.0 * (N_IMG + N_TXT) * K * N / t / 1e9, 1)}
+            del a, w
+        legs["config1_fp32_matmul_M4608"] = dict(mm, sample="full size, dequantised-operand fp32 matmul + bias, "
+                                                            "median of 3 after 1 warm-up")
+        q, k, v = [torch.randn(1, HEADS, N_IMG + N_TXT, HEAD_DIM, generator=g) for _ in range(3)]
+        t = _median_time(lambda: sdpa(q, k, v), 1, 3)
+        legs["config2_fp32_sdpa_S4608_H24"] = {"ms": round(t * 1e3, 1),
+                                               "gflops": round(4.0 * (N_IMG + N_TXT) ** 2 * HEAD_DIM * HEADS / t / 1e9, 1),
+                                               "sample": "full size, median of 3 after 1 warm-up"}
+    return legs
+
+
+def wan_cpu_baseline(cfg, S_full, S_sample=2048, reps=2):
+    """One Wan2.1-14B DiTBlock (oracle, fp32, torch SDPA) on the host cores at a REDUCED token count, extrapolated:
+    the GEMM / row-kernel part scales with S, self-attention with S^2 (measured separately), 512 text tokens kept."""
+    import torch
+
+    from oracle import wan as ow
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    c1 = dict(cfg, num_layers=1)
+    sd = ow.init_params(c1, dtype=torch.float32, seed=0)
+    P = ow.Params(sd, "plain")
+    g = torch.Generator().manual_seed(0)
+    d, H = cfg["dim"], cfg["num_heads"]
+    x, ctx, t_mod = torch.randn(1, S_sample, d, generator=g), torch.randn(1, 512, d, generator=g), \
+        torch.randn(1, 6, d, generator=g) * 0.3
+    freqs = ow.freqs_cis_3d(d // H, 1, 1, S_sample)
+    sdpa = torch.nn.functional.scaled_dot_product_attention
+    with torch.no_grad():
+        t_block = _median_time(lambda: ow.dit_block(P, 0, x, ctx, t_mod, freqs, c1, attn=sdpa), 1, reps)
+        q = torch.randn(1, H, S_sample, d // H, generator=g)
+        t_attn = _median_time(lambda: sdpa(q, q, q), 1, reps)
+    scale = S_full / S_sample
+    per_block = (t_block - t_attn) * scale + t_attn * scale * scale
+    return {"value": round(per_block * cfg["num_layers"] * 1e3, 0), "unit": "ms", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "oracle fp32 on host: one DiTBlock at %d video + 512 text tokens (%.2f s, of which self-attention "
+                      "%.2f s), EXTRAPOLATED to %d tokens (attention x%.0f, the rest x%.1f) and x%d layers"
+                      % (S_sample, t_block, t_attn, S_full, scale * scale, scale, cfg["num_layers"])}
 
 
 # L2-miss bytes per fp8_gemm_kernel launch, averaged over the 154 launches of one 19+38 step (the image/text
@@ -428,13 +578,14 @@ def main():
     for _ in range(args.warmup):
         out = runner(**inp)
     torch.cuda.synchronize()
-    with GemmTimer(torch, ops) as gt:
+    with AttnTimer(torch, ops) as at, GemmTimer(torch, ops) as gt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             out = runner(**inp)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         n_gemm, gemm_flops, gemm_secs = gt.summary()
+        n_attn, attn_flops, attn_secs = at.summary()
     assert torch.isfinite(out.float()).all().item(), "non-finite output"
     ms = (t1 - t0) * 1e3 / args.steps
 
@@ -466,12 +617,19 @@ def main():
         "step_roofline": {"algorithmic_tflop": round((gemm_fl + attn_fl) / 1e12, 2),
                           "ideal_ms": round(t_ideal * 1e3, 2), "frac": round(t_ideal * 1e3 / ms, 4)},
     }
+    result["detail"] = {"attention_in_step": {
+        "launches": n_attn, "avg_call_us": round(attn_secs / max(n_attn, 1) * 1e6, 1),
+        "tflops": round(attn_flops / max(attn_secs, 1e-12) / 1e12, 1),
+        "frac_bf16_peak": round(attn_flops / max(attn_secs, 1e-12) / PEAK_BF16, 4),
+        "ms_per_step": round(attn_secs * 1e3 / args.steps, 2)},
+        "fp8_gemm_in_step": {"ms_per_step": round(gemm_secs * 1e3 / args.steps, 2)}}
     if not args.no_micro:
-        result["detail"] = micro_benchmarks(torch, ops, dev)
+        result["detail"].update(micro_benchmarks(torch, ops, dev))
     del runner
     torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.double, args.single)
+        result["detail"]["cpu_config_legs"] = cpu_config_legs()
     print(json.dumps(result))
 
 

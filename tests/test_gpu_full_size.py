@@ -156,7 +156,12 @@ def test_full_depth_step_is_as_close_to_the_oracle_as_the_oracle_is_to_itself(de
     is not a continuous function of its input (one ulp in a row's absmax moves that row's whole quantisation
     grid), so the yardstick is measured, not assumed: the oracle is run a second time with the lowest mantissa
     bit of every 1024th latent element flipped, and the runner has to agree with the oracle as well as these
-    two oracle runs agree with each other (within 1e-3 of cosine), and to 0.99 outright."""
+    two oracle runs agree with each other (within 1e-3 of cosine), and to 0.99 outright.
+    Which part amplifies the nudge is measured too: the same nudge through the oracle's "plain" mode (bf16
+    F.linear, no e4m3 anywhere) decorrelates the output about thirty times less (0.99986 against 0.9961), so it is
+    the re-gridding of the e4m3 quantisers, not the random network, and shrinking the AdaLN gates does not remove
+    it (0.9975 with the modulation weights scaled by 0.1).  The check that can tell a wrong block from a right one
+    at this size is the teacher-forced walk over all 57 blocks in tests/test_gpu_configs.py."""
     from bench import flux_state_dict_stream
     from diffsynth_engine_amd.flux_dit import FluxDiTRunner
     from oracle import flux as oflux
@@ -180,3 +185,7 @@ def test_full_depth_step_is_as_close_to_the_oracle_as_the_oracle_is_to_itself(de
     want_nudged = oflux.flux_dit_forward(P, **nudged, num_double=19, num_single=38)
     c, floor = cos(got, want), cos(want, want_nudged)
     assert c >= 0.99 and c >= floor - 1e-3, (c, floor)
+    Pp = oflux.Params(sd, "plain")
+    plain_floor = cos(oflux.flux_dit_forward(Pp, **inp, num_double=19, num_single=38),
+                      oflux.flux_dit_forward(Pp, **nudged, num_double=19, num_single=38))
+    assert plain_floor >= 0.9995 and 1 - plain_floor < (1 - floor) / 5, (plain_floor, floor)

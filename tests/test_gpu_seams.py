@@ -86,3 +86,37 @@ def test_fp32_inputs_keep_their_dtype(dev):
     assert out.dtype == torch.float32
     want = O.sdpa(q, q, q)
     assert row_rel_err(out.cpu(), want) <= 2e-2
+
+
+def test_weight_scale_travels_with_the_module_state(dev):
+    """enable_fp8_linear -> state_dict() -> block-runner storage, and -> load_state_dict into another converted
+    module: the per-tensor scale is a buffer of the Linear (`<name>.weight_scale`), so neither path can take an
+    already scaled e4m3 weight at unit scale (wrong by 448 / absmax per layer, with no error)."""
+    from diffsynth_engine_amd import enable_fp8_linear, fp8_inference, ops
+    from diffsynth_engine_amd.flux_dit import ingest_state_dict
+
+    torch.manual_seed(3)
+    m = _Mlp().to(torch.bfloat16).to(dev)
+    enable_fp8_linear(m)
+    sd = m.state_dict()
+    assert sd["net.0.weight"].dtype == torch.float8_e4m3fn and sd["net.0.weight_scale"].dim() == 0
+    x = torch.randn(40, 256, generator=torch.Generator().manual_seed(4)).bfloat16().to(dev)
+    with fp8_inference():
+        want = m.net[0](x)
+    lin, _ = ingest_state_dict({k: sd[k] for k in sorted(sd)}, dev, scaled=True)  # bias, weight, weight_scale order
+    a_q, a_s = ops.quantize_fp8(x)
+    assert torch.equal(lin["net.0"](a_q, a_s), want)
+    # a second module converted from other weights takes this one's state in place, scale included
+    torch.manual_seed(5)
+    m2 = _Mlp().to(torch.bfloat16).to(dev)
+    with torch.no_grad():
+        m2.net[0].weight.mul_(3)
+    enable_fp8_linear(m2)
+    assert not torch.equal(m2.net[0].weight_scale, m.net[0].weight_scale)
+    m2.load_state_dict(sd)
+    with fp8_inference():
+        assert torch.equal(m2.net[0](x), want)
+    # without its scale the weight is refused rather than mis-scaled
+    del sd["net.0.weight_scale"]
+    with pytest.raises(ValueError, match="net.0"):
+        ingest_state_dict(sd, dev, scaled=True)

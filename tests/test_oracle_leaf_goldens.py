@@ -167,3 +167,35 @@ def test_reference_fp8_linear_vectors():
         d = (got.float() - y.float()).abs()
         assert (d <= y.float().abs() * 2 ** -7 + 1e-6).all(), d.max()
         assert (d > 0).float().mean().item() < 0.05
+
+
+# ---- the reference's FluxDiT.forward UNDER ITS FP8 PATCH, bf16, head dim 128 (tests/golden/make_flux_fp8_fixture.py:
+# ---- hidden 256 = 2 heads x 128, RoPE axes (16,56,56), 1 joint + 1 single block, enable_fp8_linear + fp8_inference)
+def load_fp8_d128_fixture():
+    """(state dict with float8_e4m3fn Linear weights, inputs, output) of flux_fp8_d128.safetensors."""
+    raw = load_file(os.path.join(os.path.dirname(__file__), "golden", "flux_fp8_d128.safetensors"))
+    sd = {k[len("param."):]: (v.view(torch.float8_e4m3fn) if v.dtype == torch.uint8 else v)
+          for k, v in raw.items() if k.startswith("param.")}
+    inputs = {k[len("in."):]: v for k, v in raw.items() if k.startswith("in.")}
+    return sd, inputs, raw["out"]
+
+
+def test_fp8_reference_mode_against_the_references_own_fp8_forward():
+    """The oracle's "fp8_ref" mode (bare e4m3 casts, unit scales, fp32 accumulation, bf16 rounding points of the
+    torch op sequence) against what the reference computed with torch._scaled_mm on the CPU.  With the attention
+    backend the reference used there (torch's bf16 SDPA) the oracle reproduces the reference's output BIT FOR
+    BIT: every chunk order, rounding point, bias and cast of the fp8 path is pinned.  With the oracle's own fp32
+    softmax attention the difference is that backend's bf16 arithmetic alone."""
+    sd, inputs, want = load_fp8_d128_fixture()
+    P = OF.Params(sd, "fp8_ref", heads=2, head_dim=128, axes_dim=(16, 56, 56))
+    same = OF.flux_dit_forward(P, **inputs, num_double=1, num_single=1,
+                               attn=torch.nn.functional.scaled_dot_product_attention)
+    assert same.dtype == torch.bfloat16 and torch.equal(same, want)
+    got = OF.flux_dit_forward(P, **inputs, num_double=1, num_single=1)
+    cos = torch.nn.functional.cosine_similarity(got.float().flatten(), want.float().flatten(), dim=0).item()
+    assert cos >= 0.9998, cos
+    # the scaled mode is a different function of the same weights: the fixture tells the two apart
+    Ps = OF.Params({k: (v.float() if v.dtype == torch.float8_e4m3fn else v) for k, v in sd.items()}, "fp8_scaled",
+                   heads=2, head_dim=128, axes_dim=(16, 56, 56))
+    other = OF.flux_dit_forward(Ps, **inputs, num_double=1, num_single=1)
+    assert not torch.equal(other, want)
