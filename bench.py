@@ -207,7 +207,7 @@ class GemmTimer:
 
         def timed(a_q, w_q, *args, **kw):
             M, K = a_q.shape
-            if M <= 8:
+            if M <= 8 or kw.get("qk") is not None:  # (a q/k-epilogue call goes through the grouped entry, timed there)
                 return orig(a_q, w_q, *args, **kw)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()

@@ -21,7 +21,7 @@ DSX_EARCH = -3
 DSX_ELAUNCH = -4
 DSX_ENULL = -5
 DSX_EWORKSPACE = -6
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class AttnParams(ctypes.Structure):
@@ -66,6 +66,10 @@ class GemmProblem(ctypes.Structure):
         ("rows_per_batch", c_int64),
         ("out", c_void_p), ("ldo", c_int64),
         ("M", c_int64), ("N", c_int64), ("K", c_int64),
+        ("q_norm_w", c_void_p), ("k_norm_w", c_void_p),
+        ("rope", c_void_p), ("rope_sb", c_int64), ("rope_pos0", c_int64), ("rope_rows", c_int64),
+        ("norm_eps", c_float),
+        ("qk_heads", ctypes.c_int32),
     ]
 
 

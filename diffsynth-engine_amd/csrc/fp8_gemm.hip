@@ -17,6 +17,7 @@
 // reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
 // One launch can carry two independent problems (the image- and text-stream linears of a joint
 // block): their tiles share the grid, so the small problem runs on CUs the large one leaves idle.
+#include "attn_internal.h"
 #include "common.h"
 
 namespace dsx {
@@ -46,6 +47,14 @@ struct GemmArgs {
   int rows_per_batch;
   // optional per-output-row weight scale (GEMV path only)
   const float* w_row_scale;
+  // optional RMSNorm + RoPE of the q and k heads of a packed qkv projection, applied to the bf16 result before
+  // it is stored (main kernel only): columns [0, 128*qk_heads) are q heads, the next 128*qk_heads are k heads
+  const uint16_t* qk_wq;  // (128,) bf16 or NULL
+  const uint16_t* qk_wk;
+  const float* rope;      // (rows, 64, 2) fp32 (cos, sin) or NULL; row = rope_pos0 + m % rows_per_batch
+  int64_t rope_sb;        // per batch entry m / rows_per_batch
+  int rope_pos0, qk_heads;
+  float qk_eps;
 };
 
 // Two problems in one grid: logical tiles [0, tiles of p[0]) belong to p[0], the rest to p[1].
@@ -64,6 +73,8 @@ __device__ __forceinline__ GemmArgs pick(const GemmPair& q, bool second) {
   DSX_PICK(lda); DSX_PICK(ldw); DSX_PICK(ldo); DSX_PICK(M); DSX_PICK(N); DSX_PICK(K);
   DSX_PICK(tiles_m); DSX_PICK(tiles_n); DSX_PICK(resid); DSX_PICK(gate); DSX_PICK(ldr); DSX_PICK(gate_sb);
   DSX_PICK(rows_per_batch); DSX_PICK(w_row_scale);
+  DSX_PICK(qk_wq); DSX_PICK(qk_wk); DSX_PICK(rope); DSX_PICK(rope_sb); DSX_PICK(rope_pos0); DSX_PICK(qk_heads);
+  DSX_PICK(qk_eps);
 #undef DSX_PICK
   return r;
 }
@@ -191,7 +202,11 @@ struct EpiOperands {
   float sc[2];       // [tm]: a_scale[m] * w_scale
 };
 
-template <bool RESID>
+// QK: the wave's 128 columns are one head of a packed qkv projection; q and k heads get the per-head RMSNorm and
+// the RoPE rotation (same helper and rounding points as rmsnorm_rope_qk_kernel, so the result is bit-identical to
+// that kernel run in place on the stored projection) between the LDS read-back and the global store: there the
+// 16 lanes of a DPP row hold one token's whole head row, 16 bytes each.
+template <bool RESID, bool QK>
 __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][2], const EpiOperands& e,
                                               uint8_t* wave_lds, int n_base, int m_base, int lane) {
   const int g = lane >> 5, li = lane & 31;
@@ -231,6 +246,13 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
   uint16_t* const out_lane = p.out + (int64_t)(m_base + r0) * p.ldo + n;
   const uint16_t* const res_lane = RESID ? p.resid + (int64_t)(m_base + r0) * p.ldr + n : nullptr;
   const int64_t out_step = 4 * p.ldo, res_step = 4 * p.ldr;
+  // QK pre-processing of this wave's head (wave-uniform choices): which norm weight, whether anything applies
+  const bool qk_is_q = QK && n_base < p.qk_heads * 128;
+  const bool qk_on = QK && n_base < 2 * p.qk_heads * 128;
+  const uint16_t* const qk_w = qk_is_q ? p.qk_wq : p.qk_wk;
+  u32x4 qk_wv = {0, 0, 0, 0};
+  if (QK && qk_on && qk_w) qk_wv = *reinterpret_cast<const u32x4*>(qk_w + ch * 8);
+  const bool qk_one_batch = m_base + 63 < p.rows_per_batch;  // wave-uniform: no division per row
   auto rows8 = [&](int it0, bool guarded) {
     u32x4 v[8], rv[8];
     bool ok[8];
@@ -241,6 +263,33 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
       ok[u] = !guarded || (m < p.M && col_ok);
       v[u] = *reinterpret_cast<const u32x4*>(wave_lds + ml * kEpiPitch + ch * 16);
       if (RESID && ok[u]) rv[u] = *reinterpret_cast<const u32x4*>(res_lane + (it0 + u) * res_step);
+    }
+    if (QK && qk_on) {
+      f32x4 t0[8], t1[8];
+      if (p.rope) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {  // rows past M are never stored: their table address is clamped, not predicated
+          const int m = min(m_base + (it0 + u) * 4 + r0, p.M - 1);
+          const int b = qk_one_batch ? 0 : m / p.rows_per_batch;
+          const float* cs = p.rope + (int64_t)b * p.rope_sb +
+                            (int64_t)(p.rope_pos0 + m - b * p.rows_per_batch) * 128 + ch * 8;
+          t0[u] = *reinterpret_cast<const f32x4*>(cs);
+          t1[u] = *reinterpret_cast<const f32x4*>(cs + 4);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        float rrms = 1.f;
+        if (qk_w) {
+          float ss = sumsq_chunk(v[u]);  // the 16 lanes of a DPP row hold the head row
+          ss += dpp_f32<kDppQuadXor1>(ss);
+          ss += dpp_f32<kDppQuadXor2>(ss);
+          ss += dpp_f32<kDppRowRor4>(ss);
+          ss += dpp_f32<kDppRowRor8>(ss);
+          rrms = rsqrtf(ss * (1.0f / 128) + p.qk_eps);
+        }
+        v[u] = norm_rope_regs(v[u], qk_w != nullptr, rrms, qk_wv, p.rope != nullptr, t0[u], t1[u]);
+      }
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
@@ -305,7 +354,7 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
   }
 }
 
-template <bool RESID>
+template <bool RESID, bool QK>
 __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // Both problems' arguments are fetched together with the tile counts, in one round of scalar loads, and the
@@ -495,7 +544,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   // are issued -- the two waves of a SIMD then overlap one's conversion with the other's last MFMAs.
   epi.sc[0] *= w_scale_raw;
   epi.sc[1] *= w_scale_raw;
-  store_ct_lds<RESID>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 64, lane);
+  store_ct_lds<RESID, QK>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 64, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -656,9 +705,11 @@ static int gemm_set_attributes() {
   using namespace dsx;
   static PerDeviceOnce once;
   return per_device_once(once, [](int) {
-    if (hipFuncSetAttribute((const void*)fp8_gemm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute((const void*)fp8_gemm_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kMainLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             kMainLdsBytes) != hipSuccess ||
         hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
@@ -679,7 +730,7 @@ static bool gemm_main_kernel_ok(dsx::GemmArgs& p) {
   return p.M > 8 && !p.w_row_scale && (p.K % 128) == 0 && vec_ok;
 }
 
-// One launch of the main kernel over one or two problems (both with or both without a residual).
+// One launch of the main kernel over one or two problems (of the same kind: plain, residual or qk epilogue).
 static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStream_t st) {
   using namespace dsx;
   GemmPair q;
@@ -689,9 +740,11 @@ static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStre
   q.total = q.total0 + (p1 ? p1->tiles_m * p1->tiles_n : 0);
   const int grid = ((q.total + 7) / 8) * 8;
   if (p0.resid)
-    fp8_gemm_kernel<true><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<true, false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+  else if (p0.qk_heads > 0)
+    fp8_gemm_kernel<false, true><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   else
-    fp8_gemm_kernel<false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<false, false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
@@ -744,6 +797,11 @@ static int gemm_fill(dsx::GemmArgs& p, const void* a, int64_t lda, const void* w
   p.ldr = p.gate_sb = 0;
   p.rows_per_batch = 1;
   p.w_row_scale = nullptr;
+  p.qk_wq = p.qk_wk = nullptr;
+  p.rope = nullptr;
+  p.rope_sb = 0;
+  p.rope_pos0 = p.qk_heads = 0;
+  p.qk_eps = 0.f;
   return DSX_OK;
 }
 
@@ -802,6 +860,28 @@ static int problem_fill(dsx::GemmArgs& p, const dsx_gemm_problem& d) {
   } else if (d.gate) {
     return DSX_ENULL;  // a gate without a residual is not an operation of the path
   }
+  if (d.qk_heads != 0) {
+    // the q/k epilogue lives in the 256x256-tile kernel only, whose waves own whole 128-column heads
+    if (d.qk_heads < 0 || d.resid || d.M <= 0 || 2 * (int64_t)d.qk_heads * 128 > d.N) return DSX_EBADSHAPE;
+    if (d.rows_per_batch <= 0 || d.rows_per_batch > (1 << 30)) return DSX_EBADSHAPE;
+    if (((uintptr_t)d.q_norm_w & 15) || ((uintptr_t)d.k_norm_w & 15) || ((uintptr_t)d.rope & 15) || (d.rope_sb & 3))
+      return DSX_EALIGN;
+    if (d.rope) {
+      const int64_t batches = (d.M + d.rows_per_batch - 1) / d.rows_per_batch;
+      const int64_t last = d.rope_pos0 + (d.M < d.rows_per_batch ? d.M : d.rows_per_batch);
+      if (d.rope_pos0 < 0 || d.rope_pos0 > (1 << 30) || d.rope_rows < last) return DSX_EBADSHAPE;
+      if (batches > 1 && d.rope_sb != 0 && d.rope_sb < d.rope_rows * 128) return DSX_EBADSHAPE;
+    }
+    p.qk_wq = (const uint16_t*)d.q_norm_w;
+    p.qk_wk = (const uint16_t*)d.k_norm_w;
+    p.rope = d.rope;
+    p.rope_sb = d.rope_sb;
+    p.rope_pos0 = (int)d.rope_pos0;
+    p.qk_heads = d.qk_heads;
+    p.qk_eps = d.norm_eps;
+    p.rows_per_batch = (int)d.rows_per_batch;
+    if (!gemm_main_kernel_ok(p)) return DSX_EBADSHAPE;
+  }
   return DSX_OK;
 }
 
@@ -822,7 +902,8 @@ extern "C" int dsx_fp8_gemm_grouped(const dsx_gemm_problem* problems, int count,
   while (i < count) {
     if (args[i].M == 0) { ++i; continue; }
     // pair neighbours that both run on the main kernel and agree on having a residual
-    if (i + 1 < count && main_ok[i] && main_ok[i + 1] && (args[i].resid != nullptr) == (args[i + 1].resid != nullptr)) {
+    if (i + 1 < count && main_ok[i] && main_ok[i + 1] && (args[i].resid != nullptr) == (args[i + 1].resid != nullptr) &&
+        (args[i].qk_heads > 0) == (args[i + 1].qk_heads > 0)) {
       const int rc = launch_main(args[i], &args[i + 1], st);
       if (rc != DSX_OK) return rc;
       i += 2;

@@ -62,14 +62,16 @@ class _Linear:
         uq, us = ops.quantize_weight_fp8(u, scaled=True)
         self.loras.append((dq, ds, uq, (us * coef).float()))
 
-    def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
+    def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None, qk=None):
         """Keyword arguments of ``ops.fp8_gemm`` for this layer applied to ``a_q``."""
         return dict(a_q=a_q, w_q=self.w, a_scale=a_s if self.s is not None else None, w_scale=self.s, bias=self.b,
-                    out=out, resid=resid, gate=gate, rows_per_batch=rows_per_batch)
+                    out=out, resid=resid, gate=gate, rows_per_batch=rows_per_batch, qk=qk)
 
-    def __call__(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None):
+    def __call__(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None, qk=None):
         if not self.loras:
-            return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch))
+            return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch, qk))
+        if qk is not None:  # the low-rank terms are added after the main product: q/k can only be prepared after them
+            raise ValueError("a LoRA on a qkv projection needs qk_prep='attention'")
         lows = []
         for dq, ds, uq, us in self.loras:
             hq, hs = ops.quantize_fp8(ops.fp8_gemm(a_q, dq, a_s, ds, None), scaled=True)
@@ -147,9 +149,16 @@ class FluxDiTRunner:
     from the checkpoint (``x_embedder.weight``); heads are 128 wide (``heads`` = hidden / 128 unless given)."""
 
     def __init__(self, state_dict, num_double: int = 19, num_single: int = 38, scaled: bool = True,
-                 device="cuda:0", heads: Optional[int] = None, axes_dim=AXES_DIM):
+                 device="cuda:0", heads: Optional[int] = None, axes_dim=AXES_DIM, qk_prep: str = "gemm"):
         self.device = torch.device(device)
         self.scaled = scaled
+        # Where the per-head RMSNorm and the RoPE rotation of q and k happen (flux_dit.py:165-171,179-180,297-301):
+        # "gemm": in the epilogue of the qkv projection, on the tile the GEMM is about to store (no pass of its
+        # own; the attention call is then plain); "attention": requested from the attention entry point (k in one
+        # row pass into scratch, q as the attention kernel loads it).  Same arithmetic, same bits.
+        if qk_prep not in ("gemm", "attention"):
+            raise ValueError("qk_prep must be 'gemm' or 'attention', got %r" % (qk_prep,))
+        self.qk_prep = qk_prep
         self.num_double, self.num_single = num_double, num_single
         self.lin, other = ingest_state_dict(state_dict, self.device, scaled)
         self.norm_w: Dict[str, torch.Tensor] = {}
@@ -207,6 +216,13 @@ class FluxDiTRunner:
         projections are stacked at construction and take no LoRA here."""
         self.lin[name].add_lora(down, up, coef)
 
+    def _qk_in_gemm(self, rows, *layers) -> bool:
+        """q/k are prepared in the GEMM epilogue unless a LoRA rides on one of the projections (its low-rank
+        terms are added after the main product, so the projection is complete only after them) or a problem is
+        outside what the tile kernel that carries the epilogue takes (more than 8 rows, K a multiple of 128)."""
+        return (self.qk_prep == "gemm" and not any(L.loras for L in layers) and min(rows) > 8
+                and all(L.k % 128 == 0 and L.n % 8 == 0 for L in layers))
+
     # ------------------------------------------------------------------ small helpers
     def _linear_bf16(self, x: torch.Tensor, name: str) -> torch.Tensor:
         """quantise + GEMM for a bf16 activation (embedders and M=1 conditioning projections)."""
@@ -261,11 +277,18 @@ class FluxDiTRunner:
         St = txt.shape[1]
         ma, mb = mod_a.chunk(6, dim=1), mod_b.chunk(6, dim=1)
         L = self.lin
+        nw = self.norm_w
         qa, sa = self._modulate_q(img, ma[1], ma[0])
         qb, sb = self._modulate_q(txt, mb[1], mb[0])
-        qkv_a, qkv_b = _gemm_pair(L[pre + "attn.a_to_qkv"], dict(a_q=qa.view(-1, d), a_s=sa),
-                                  L[pre + "attn.b_to_qkv"], dict(a_q=qb.view(-1, d), a_s=sb))
-        nw = self.norm_w
+        in_gemm = self._qk_in_gemm((B * Si, B * St), L[pre + "attn.a_to_qkv"], L[pre + "attn.b_to_qkv"])
+        qk_a = qk_b = None
+        if in_gemm:  # text rows take RoPE rows [0, St), image rows [St, St + Si) of every batch entry
+            qk_a = dict(heads=HEADS, q_norm_w=nw[pre + "attn.norm_q_a"], k_norm_w=nw[pre + "attn.norm_k_a"], rope=rope,
+                        pos0=St, eps=EPS)
+            qk_b = dict(heads=HEADS, q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"], rope=rope,
+                        pos0=0, eps=EPS)
+        qkv_a, qkv_b = _gemm_pair(L[pre + "attn.a_to_qkv"], dict(a_q=qa.view(-1, d), a_s=sa, rows_per_batch=Si, qk=qk_a),
+                                  L[pre + "attn.b_to_qkv"], dict(a_q=qb.view(-1, d), a_s=sb, rows_per_batch=St, qk=qk_b))
         qkv_a = qkv_a.view(B, Si, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         qkv_b = qkv_b.view(B, St, 3 * HEADS, HEAD_DIM).transpose(1, 2)
         # With one batch entry the text and image rows of an intermediate share one [text; image] buffer, so
@@ -280,12 +303,17 @@ class FluxDiTRunner:
             o_a = torch.empty((B, Si, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=img.device)
         qb_, kb_, vb_ = qkv_b[:, :HEADS], qkv_b[:, HEADS:2 * HEADS], qkv_b[:, 2 * HEADS:]
         qa_, ka_, va_ = qkv_a[:, :HEADS], qkv_a[:, HEADS:2 * HEADS], qkv_a[:, 2 * HEADS:]
-        # joint attention over [text; image] rows with the per-stream q/k RMSNorm weights and the RoPE table
-        ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, rope=rope,
-                           q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
-                           q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
-                           out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2),
-                           score_bound=self.score_bound.get(pre, 0.0))
+        # joint attention over [text; image] rows; q and k either arrive prepared from the GEMM epilogue or go in
+        # with the per-stream RMSNorm weights and the RoPE table
+        if in_gemm:
+            ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2),
+                               score_bound=self.score_bound.get(pre, 0.0))
+        else:
+            ops.attention_bhsd(qb_, kb_, vb_, q2=qa_, k2=ka_, v2=va_, rope=rope,
+                               q_norm_w=nw[pre + "attn.norm_q_b"], k_norm_w=nw[pre + "attn.norm_k_b"],
+                               q2_norm_w=nw[pre + "attn.norm_q_a"], k2_norm_w=nw[pre + "attn.norm_k_a"], eps=EPS,
+                               out=o_b.transpose(1, 2), out2=o_a.transpose(1, 2),
+                               score_bound=self.score_bound.get(pre, 0.0))
         # The two streams run the same sequence on different weights (flux_dit.py:226-234): out-projection +
         # gated residual, LN-modulate, MLP + gated residual.  Each pair of linears goes out as one grouped
         # submission so that the 512-token text problem runs beside the image problem instead of after it.
@@ -325,13 +353,19 @@ class FluxDiTRunner:
         L = self.lin
         shift, scale, gate = mod.chunk(3, dim=1)
         q, sc = self._modulate_q(x, scale, shift)
-        h = L[pre + "to_qkv_mlp"](q.view(-1, d), sc)  # (B*S, 7d): [q | k | v | mlp]
+        nw = self.norm_w
+        in_gemm = self._qk_in_gemm((B * S,), L[pre + "to_qkv_mlp"])
+        qk = dict(heads=HEADS, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"], rope=rope, pos0=0,
+                  eps=EPS) if in_gemm else None
+        h = L[pre + "to_qkv_mlp"](q.view(-1, d), sc, rows_per_batch=S, qk=qk)  # (B*S, 7d): [q | k | v | mlp]
         att = torch.empty((B, S, HEADS, HEAD_DIM), dtype=torch.bfloat16, device=x.device)
         qkv = h.view(B, S, 7 * d)[:, :, : 3 * d].unflatten(2, (3 * HEADS, HEAD_DIM)).transpose(1, 2)
-        nw = self.norm_w
         q_, k_, v_ = qkv[:, :HEADS], qkv[:, HEADS:2 * HEADS], qkv[:, 2 * HEADS:]
-        ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
-                           eps=EPS, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
+        if in_gemm:
+            ops.attention_bhsd(q_, k_, v_, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
+        else:
+            ops.attention_bhsd(q_, k_, v_, rope=rope, q_norm_w=nw[pre + "norm_q_a"], k_norm_w=nw[pre + "norm_k_a"],
+                               eps=EPS, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
         # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
         # parts and emits the e4m3 operand of proj_out with its per-token scale
         if self.scaled:

@@ -87,8 +87,12 @@ def quantize_weight_fp8(w: torch.Tensor, scaled: bool = True):
 
 
 def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, resid=None, gate=None,
-                  rows_per_batch=None):
-    """Validate one GEMM and describe it as a ``dsx_gemm_problem``; returns (problem, out, keep-alive refs)."""
+                  rows_per_batch=None, qk=None):
+    """Validate one GEMM and describe it as a ``dsx_gemm_problem``; returns (problem, out, keep-alive refs).
+
+    ``qk``: optional dict(heads=H, q_norm_w=, k_norm_w=, rope=(B|1, S, 64, 2) fp32 table or None, pos0=, eps=) for a
+    packed qkv projection: per-head RMSNorm + RoPE of the q and k heads in the GEMM's epilogue (rows_per_batch =
+    tokens per batch entry; token t of an entry takes table row pos0 + t)."""
     _require_cuda(a_q, w_q)
     if a_q.dtype != FP8 or w_q.dtype != FP8:
         raise ValueError("fp8_gemm expects float8_e4m3fn operands")
@@ -125,17 +129,38 @@ def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, res
         a=_ptr(a_q), lda=a_q.stride(0), w=_ptr(w_q), ldw=w_q.stride(0), a_scale=_ptr(a_scale), w_scale=_ptr(w_scale),
         bias=_ptr(bias), resid=_ptr(resid), ldr=resid.stride(0) if resid is not None else 0, gate=_ptr(gate),
         gate_sb=gate_sb, rows_per_batch=(rows_per_batch or max(M, 1)), out=_ptr(out), ldo=out.stride(0), M=M, N=N, K=K)
-    return prob, out, (a_q, w_q, a_scale, w_scale, bias, resid, gate)
+    keep = [a_q, w_q, a_scale, w_scale, bias, resid, gate]
+    if qk is not None:
+        if resid is not None:
+            raise ValueError("fp8_gemm: the q/k epilogue and the residual epilogue exclude each other")
+        wq, wk, rope = qk.get("q_norm_w"), qk.get("k_norm_w"), qk.get("rope")
+        wq = None if wq is None else wq.to(_BF16).contiguous()
+        wk = None if wk is None else wk.to(_BF16).contiguous()
+        prob.q_norm_w, prob.k_norm_w = _ptr(wq), _ptr(wk)
+        prob.qk_heads, prob.norm_eps = int(qk["heads"]), float(qk.get("eps", 1e-6))
+        if rope is not None:
+            if rope.dtype != torch.float32 or rope.dim() != 4 or rope.shape[2:] != (64, 2):
+                raise ValueError("rope table must be fp32 (B|1, S, 64, 2)")
+            rope = rope.contiguous()
+            prob.rope, prob.rope_rows = _ptr(rope), rope.shape[1]
+            prob.rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
+            prob.rope_pos0 = int(qk.get("pos0", 0))
+        keep += [wq, wk, rope]
+    return prob, out, tuple(keep)
 
 
 def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor] = None,
              w_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
              out: Optional[torch.Tensor] = None, resid: Optional[torch.Tensor] = None,
-             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None) -> torch.Tensor:
+             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None, qk=None) -> torch.Tensor:
     """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3.
 
     With ``resid`` (M,N) the gated residual is fused: out = resid + gate * that, gate (B,N) or None,
-    rows_per_batch = rows of a per batch entry (default: all M rows share gate row 0)."""
+    rows_per_batch = rows of a per batch entry (default: all M rows share gate row 0).
+    With ``qk`` (see _gemm_problem) the q and k heads of a packed qkv projection leave normalised and rotated."""
+    if qk is not None:
+        return fp8_gemm_grouped([dict(a_q=a_q, w_q=w_q, a_scale=a_scale, w_scale=w_scale, bias=bias, out=out,
+                                      rows_per_batch=rows_per_batch, qk=qk)])[0]
     pr, out, _keep = _gemm_problem(a_q, w_q, a_scale, w_scale, bias, out, resid, gate, rows_per_batch)
     lib = _lib.load()
     if resid is None:

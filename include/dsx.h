@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define DSX_ABI_VERSION 3
+#define DSX_ABI_VERSION 4
 
 enum {
   DSX_OK = 0,
@@ -107,7 +107,7 @@ int dsx_fp8_gemm_gated_residual(const void* a, int64_t lda, const void* w, int64
  * Up to DSX_GEMM_GROUP_MAX independent FP8 GEMMs submitted together.  Each problem is exactly
  * dsx_fp8_gemm (resid == NULL) or dsx_fp8_gemm_gated_residual (resid != NULL) with the same argument
  * meaning and the same checks; neighbouring problems that both qualify for the 256x256-tile kernel
- * and agree on having a residual share ONE launch, so a small problem runs on compute units a
+ * and are of the same kind (plain, residual, q/k epilogue) share ONE launch, so a small problem runs on compute units a
  * large one leaves idle.  The reference issues the image-stream and text-stream linears of a joint
  * block as separate F.linear calls (diffsynth_engine/models/flux/flux_dit.py:165-171,190-194,
  * 227-235); this is those pairs.  All problems are validated before anything is launched.
@@ -124,6 +124,20 @@ typedef struct dsx_gemm_problem {
   int64_t rows_per_batch;              /* >= 1 when resid is given */
   void* out; int64_t ldo;              /* (M,N) bf16 */
   int64_t M, N, K;
+  /* Optional (qk_heads > 0; resid must be NULL): the problem is a packed qkv projection whose columns
+   * [0, 128*qk_heads) are q heads and [128*qk_heads, 256*qk_heads) k heads (further columns: v, ... untouched),
+   * and the per-head RMSNorm (q_norm_w / k_norm_w, bf16 (128,), either may be NULL) and the RoPE rotation
+   * (rope: fp32 (cos, sin) table as in dsx_attn_params, NULL = none) are applied to those heads in the epilogue,
+   * after bias and the bf16 rounding of the projection and before the store: bit-identical to dsx_rmsnorm_rope_qk
+   * run in place on the stored projection.  Row m is token m % rows_per_batch of batch entry m / rows_per_batch and
+   * takes table row rope_pos0 + m % rows_per_batch (+ rope_sb per batch entry); rope_rows rows per entry exist.
+   * Replaces norm_q / norm_k and apply_rope at models/flux/flux_dit.py:165-171,179-180,297-301 (RMSNorm:
+   * models/basic/transformer_helper.py:73-78) without a pass of its own.  Needs the shape the 256x256-tile kernel
+   * takes (M > 8, K % 128 == 0, N % 8 == 0, 16-byte aligned out), DSX_EBADSHAPE otherwise. */
+  const void* q_norm_w; const void* k_norm_w;
+  const float* rope; int64_t rope_sb, rope_pos0, rope_rows;
+  float norm_eps;
+  int32_t qk_heads;
 } dsx_gemm_problem;
 int dsx_fp8_gemm_grouped(const dsx_gemm_problem* problems, int count, void* stream);
 

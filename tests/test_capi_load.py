@@ -32,7 +32,7 @@ def test_abi_version_and_strerror():
     from diffsynth_engine_amd import _lib
 
     lib = _lib.load()
-    assert lib.dsx_abi_version() == 3
+    assert lib.dsx_abi_version() == 4
     assert _lib.strerror(0) == "ok"
     for code in (-1, -2, -3, -4, -5, -6):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
@@ -220,3 +220,29 @@ def test_gemm_refuses_leading_dimensions_beyond_its_32_bit_tile_offsets():
     assert lib.dsx_fp8_gemm(p16, 128, p16, big, None, None, None, p16, 256, 16, 256, 128, None) == _lib.DSX_EBADSHAPE
     n = 1 << 30  # 2^24 x 2^24 tiles of 64 x 64
     assert lib.dsx_fp8_gemm(p16, 128, p16, 128, None, None, None, p16, n, n, n, 128, None) == _lib.DSX_EBADSHAPE
+
+
+def test_gemm_problem_struct_layout_and_qk_epilogue_checks():
+    """dsx_gemm_problem: 17 eight-byte fields, then the q/k epilogue's two weight pointers, table pointer, three
+    int64, a float and an int32.  The q/k epilogue is refused (before any launch) with a residual, with fewer columns
+    than 2 * heads * 128, with a RoPE table that ends before the last token's row, and outside the tile kernel's shapes."""
+    from diffsynth_engine_amd import _lib
+
+    assert ctypes.sizeof(_lib.GemmProblem) == 17 * 8 + 2 * 8 + 8 + 3 * 8 + 4 + 4
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(1 << 12)
+    p16 = (ctypes.addressof(buf) + 15) & ~15
+
+    def problem(**kw):
+        base = dict(a=p16, lda=128, w=p16, ldw=128, out=p16, ldo=512, M=64, N=512, K=128, rows_per_batch=64,
+                    qk_heads=2, rope=p16, rope_rows=64, norm_eps=1e-6)
+        base.update(kw)
+        return (_lib.GemmProblem * 1)(_lib.GemmProblem(**base))
+
+    assert lib.dsx_fp8_gemm_grouped(problem(resid=p16, ldr=512), 1, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_fp8_gemm_grouped(problem(qk_heads=3), 1, None) == _lib.DSX_EBADSHAPE       # 768 columns needed
+    assert lib.dsx_fp8_gemm_grouped(problem(rope_rows=63), 1, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_fp8_gemm_grouped(problem(rope_pos0=1), 1, None) == _lib.DSX_EBADSHAPE       # rows 1..64 of 64
+    assert lib.dsx_fp8_gemm_grouped(problem(K=144, lda=144, ldw=144), 1, None) == _lib.DSX_EBADSHAPE  # K % 128
+    assert lib.dsx_fp8_gemm_grouped(problem(M=8), 1, None) == _lib.DSX_EBADSHAPE               # the GEMV path has none
+    assert lib.dsx_fp8_gemm_grouped(problem(rope=p16 + 4), 1, None) == _lib.DSX_EALIGN

@@ -61,6 +61,42 @@ def test_deeper_step_matches_oracle(dev):
     assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
 
 
+def test_qk_prep_in_the_gemm_epilogue_agrees_with_qk_prep_by_the_attention_call(dev):
+    """The two places the runner can normalise and rotate q and k: the qkv GEMM's epilogue (bit-identical to the
+    in-place row kernel, tests/test_gpu_quant_gemm.py) and the attention entry point (k by the row kernel, q inside
+    the attention kernel, where the sum of squares is taken in another order: an occasional last-bit difference of
+    the reciprocal rms).  One joint and one single block on the same inputs, one batch entry and two (the RoPE row
+    restarts per entry): outputs agree far inside the one-block bar."""
+    from diffsynth_engine_amd import ops
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+    from oracle import dit_ops as O
+
+    sd = {k: v.to(dev) for k, v in oflux.init_params(1, 1, dtype=torch.bfloat16, seed=17, bias_std=0.02).items()}
+    for k in sd:
+        if "norm_q" in k or "norm_k" in k:
+            sd[k] = (1 + 0.2 * torch.randn(128, generator=torch.Generator().manual_seed(len(k)))).bfloat16().to(dev)
+    a = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev, qk_prep="gemm")
+    b = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev, qk_prep="attention")
+    St, side = 40, 12
+    ids = torch.cat([torch.zeros(1, St, 3), oflux.image_ids(2 * side, 2 * side, 1, "cpu", torch.float32)], dim=1)
+    g = torch.Generator().manual_seed(18)
+    for B in (1, 2):
+        rope = ops.rope_table_from_freqs(O.rope_table(ids.repeat(B, 1, 1) * torch.arange(1, B + 1).view(B, 1, 1),
+                                                      oflux.AXES_DIM, oflux.THETA)).to(dev)
+        img = torch.randn(B, side * side, 3072, generator=g).bfloat16().to(dev)
+        txt = torch.randn(B, St, 3072, generator=g).bfloat16().to(dev)
+        cond = torch.randn(B, 3072, generator=g).bfloat16().to(dev)
+        mods = a._modulations(cond)
+        outs = [R._joint_block(0, img, txt, mods["blocks.0.norm1_a.linear"], mods["blocks.0.norm1_b.linear"], rope)
+                for R in (a, b)]
+        assert _cos(outs[0][0], outs[1][0]) >= 0.99995 and _cos(outs[0][1], outs[1][1]) >= 0.99995
+        x = torch.cat([txt, img], dim=1)
+        xa, xb = [R._single_block(0, x, mods["single_blocks.0.norm.linear"], rope) for R in (a, b)]
+        assert _cos(xa, xb) >= 0.99995, _cos(xa, xb)
+    with pytest.raises(ValueError):
+        FluxDiTRunner(sd, 1, 1, device=dev, qk_prep="elsewhere")
+
+
 def test_blocks_teacher_forced_against_oracle(dev):
     """Each block fed the oracle's own inputs (no error carried between blocks): joint block and single block
     outputs against the CPU oracle.  One block holds 4-5 chained e4m3 quantisations, hence 0.9995 rather than 1."""

@@ -234,3 +234,63 @@ def test_fp8_gemm_grouped_rejects_bad_arguments(dev):
     bad["gate"] = torch.ones(1, 64, dtype=torch.bfloat16, device=dev)   # gate without residual
     with pytest.raises(ValueError):
         ops.fp8_gemm_grouped([ok, bad])
+
+
+@pytest.mark.parametrize("M,heads,extra,batch,use_rope,use_norm", [
+    (4608, 24, 3072, 1, True, True),     # a Flux joint-block qkv projection: [q | k | v]
+    (1000, 2, 256 + 1024, 1, True, True),  # ragged last tile row; [q | k | v | mlp] like the single block
+    (600, 3, 384, 2, True, True),        # two batch entries of 300 tokens: the table row restarts at 300
+    (300, 2, 256, 1, False, True),       # RMSNorm only
+    (300, 2, 256, 1, True, False),       # RoPE only
+])
+def test_qk_epilogue_equals_the_in_place_row_kernel(dev, M, heads, extra, batch, use_rope, use_norm):
+    """The qkv GEMM whose epilogue normalises and rotates the q and k heads == the plain GEMM followed by
+    dsx_rmsnorm_rope_qk in place on its output, bit for bit; v (and mlp) columns untouched."""
+    from diffsynth_engine_amd import ops
+
+    K, N = 512, 2 * heads * 128 + extra
+    g = torch.Generator().manual_seed(M + heads)
+    x = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(dev)
+    bias = torch.randn(N, generator=g).bfloat16().to(dev)
+    S, pos0 = M // batch, 7
+    rope = None
+    if use_rope:
+        ang = torch.rand(batch, pos0 + S, 64, generator=g) * 6.28
+        rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).float().to(dev)
+    wq = (1 + 0.2 * torch.randn(128, generator=g)).bfloat16().to(dev) if use_norm else None
+    wk = (1 + 0.2 * torch.randn(128, generator=g)).bfloat16().to(dev) if use_norm else None
+    wq8, ws = ops.quantize_weight_fp8(w)
+    xq, xs = ops.quantize_fp8(x)
+    plain = ops.fp8_gemm(xq, wq8, xs, ws, bias)
+    want = ops.rmsnorm_rope_qk(plain.clone().view(batch, S, N), heads, heads, wq, wk, rope, pos0=pos0).view(M, N)
+    got = ops.fp8_gemm(xq, wq8, xs, ws, bias, rows_per_batch=S,
+                       qk=dict(heads=heads, q_norm_w=wq, k_norm_w=wk, rope=rope, pos0=pos0, eps=1e-6))
+    assert torch.equal(got, want)
+    assert torch.equal(got[:, 2 * heads * 128:], plain[:, 2 * heads * 128:])
+    assert not torch.equal(got[:, : 2 * heads * 128], plain[:, : 2 * heads * 128])
+
+
+def test_qk_epilogue_on_a_grouped_text_and_image_pair(dev):
+    """Two problems in one launch, each with its own norm weights and its own first RoPE row (text rows first, then
+    image rows), as the joint block submits them."""
+    from diffsynth_engine_amd import ops
+
+    heads, K, St, Si = 2, 256, 40, 300
+    N = 3 * heads * 128
+    g = torch.Generator().manual_seed(3)
+    ang = torch.rand(1, St + Si, 64, generator=g) * 6.28
+    rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).float().to(dev)
+    probs, wants = [], []
+    for rows, pos0 in ((Si, St), (St, 0)):
+        x = torch.randn(rows, K, generator=g).bfloat16().to(dev)
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(dev)
+        wq, wk = [(1 + 0.2 * torch.randn(128, generator=g)).bfloat16().to(dev) for _ in range(2)]
+        w8, ws = ops.quantize_weight_fp8(w)
+        xq, xs = ops.quantize_fp8(x)
+        plain = ops.fp8_gemm(xq, w8, xs, ws, None)
+        wants.append(ops.rmsnorm_rope_qk(plain.view(1, rows, N), heads, heads, wq, wk, rope, pos0=pos0).view(rows, N))
+        probs.append(dict(a_q=xq, w_q=w8, a_scale=xs, w_scale=ws, rows_per_batch=rows,
+                          qk=dict(heads=heads, q_norm_w=wq, k_norm_w=wk, rope=rope, pos0=pos0)))
+    outs = ops.fp8_gemm_grouped(probs)
+    assert torch.equal(outs[0], wants[0]) and torch.equal(outs[1], wants[1])
