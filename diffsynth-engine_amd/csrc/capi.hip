@@ -25,3 +25,58 @@ extern "C" int dsx_check_device(void) {
   if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return DSX_EARCH;
   return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? DSX_OK : DSX_EARCH;
 }
+
+// ---- on-box microbenchmark of the matrix pipe: MFMAs on register operands in a loop, no memory traffic --------
+// What the chip sustains with nothing but matrix instructions in flight, for the operand bits the caller supplies
+// (all-zero operands run at the full clock; random bits draw more power and the clock management lowers the clock).
+namespace dsx {
+template <int KIND>
+__global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __restrict__ bits, int64_t iters,
+                                                           float* __restrict__ sink) {
+  // eight operand dwords per lane (bf16: 4 + 4 are used; fp8: 8 + 8), the same for every workgroup
+  uint32_t r[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r[i] = bits[i * 256 + threadIdx.x];
+  f32x16 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+  for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {  // four independent accumulators
+      if (KIND == 0) {
+        const u32x4 a = {r[0], r[1], r[2], r[3]}, b = {r[4 + t], r[5 + t], r[6 + t], r[7 + t]};
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                         acc[t], 0, 0, 0);
+      } else {
+        const i32x8 a = {(int)r[0], (int)r[1], (int)r[2], (int)r[3], (int)r[4], (int)r[5], (int)r[6], (int)r[7]};
+        const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
+                         (int)r[15 - (t >> 1)]};
+        acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
+      }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s += acc[t][e];
+  if (s == 12345.678f) sink[0] = s;  // keeps the loop alive; never true for the inputs of the probe
+}
+}  // namespace dsx
+
+extern "C" int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_t iters, int32_t workgroups,
+                                      void* sink, int64_t* flops_out, void* stream) {
+  if (!operand_bits || !sink) return DSX_ENULL;
+  if ((kind != 0 && kind != 1) || iters <= 0 || iters > (1ll << 32) || workgroups <= 0 || workgroups > (1 << 20))
+    return DSX_EBADSHAPE;
+  if ((uintptr_t)operand_bits & 3) return DSX_EALIGN;
+  const dim3 grid((unsigned)workgroups), block(256);
+  if (kind == 0)
+    dsx::mfma_ceiling_kernel<0><<<grid, block, 0, (hipStream_t)stream>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+  else
+    dsx::mfma_ceiling_kernel<1><<<grid, block, 0, (hipStream_t)stream>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * 4 * (kind == 0 ? 2ll * 32 * 32 * 16 : 2ll * 32 * 32 * 64);
+  return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+}

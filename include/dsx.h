@@ -321,6 +321,17 @@ int dsx_concat_gelu_tanh(const void* prefix, int64_t ldp, int64_t Dp, const void
 int dsx_flow_match_euler_step(const void* latents, const void* v, float dt, void* out, int64_t n,
                               int is_fp32, void* stream);
 
+/*
+ * Diagnostic, no counterpart in the reference: the on-box microbenchmark behind the roofline denominators.
+ * Launches `workgroups` workgroups of four wavefronts that each run `iters` x 4 MFMAs (kind 0:
+ * v_mfma_f32_32x32x16_bf16, kind 1: v_mfma_f32_32x32x64 on e4m3 operands) on register operands taken from
+ * operand_bits (16 x 256 dwords, device memory; all zero or random, which changes power draw and with it the clock),
+ * with no memory traffic inside the loop.  *flops_out (host memory, may be NULL) receives the flops of the launch; the
+ * caller times it.  sink: one device float (never written for finite inputs).
+ */
+int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_t iters, int32_t workgroups, void* sink,
+                           int64_t* flops_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
