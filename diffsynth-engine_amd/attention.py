@@ -54,13 +54,10 @@ def wan_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, attn_impl: Optional[str] = "mi355x",
               attn_mask: Optional[torch.Tensor] = None, scale: Optional[float] = None) -> torch.Tensor:
-    """(B,S,H,D) in and out."""
-    if attn_impl not in SUPPORTED_IMPLEMENTATIONS:
-        raise ValueError(f"attn_impl must be one of {SUPPORTED_IMPLEMENTATIONS}, but got '{attn_impl}'")
-    if attn_impl == "sdpa":
-        o = nn.functional.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
-                                                       attn_mask=attn_mask, scale=scale)
-        return o.transpose(1, 2)
+    """(B,S,H,D) in and out.  This package computes with its own kernels only: the reference's other backends
+    (models/basic/attention.py:42-66) are the reference's to run, and asking for one here is a ValueError."""
+    if attn_impl != "mi355x":
+        raise ValueError(f"attn_impl must be 'mi355x' here, but got '{attn_impl}'")
     if attn_mask is not None:
         raise ValueError("attn_impl='mi355x' does not take an attention mask")
     B, Sq, H, D = q.shape
