@@ -555,12 +555,12 @@ def wan_cpu_baseline(cfg, S_full, S_sample=2048, reps=2):
                       % (S_sample, t_block, t_attn, S_full, scale * scale, scale, cfg["num_layers"])}
 
 
-# L2-miss bytes per fp8_gemm_kernel launch, averaged over the 154 launches of one 19+38 step (the image/text
-# pairs of the joint blocks share a launch): rocprofv3 --pmc FETCH_SIZE (367.6 MB) plus --pmc WRITE_SIZE
-# (87.4 MB), each scaled by what the same counter reads for the 256 MiB copy of --calibrate-copy (FETCH_SIZE
+# L2-miss bytes per fp8_gemm_kernel launch, averaged over the 152 block-GEMM launches of one 19+38 step (the
+# image/text pairs of the joint blocks share a launch): rocprofv3 --pmc FETCH_SIZE (380.3 MB) plus --pmc WRITE_SIZE
+# (88.5 MB), each scaled by what the same counter reads for the 256 MiB copy of --calibrate-copy (FETCH_SIZE
 # counts half the copied bytes, WRITE_SIZE all of them); profiles/flux_step_hbm_traffic_pmc.txt holds the
 # per-shape figures.
-GEMM_TRAFFIC_BYTES = 455.0e6
+GEMM_TRAFFIC_BYTES = 468.8e6
 
 
 def main():

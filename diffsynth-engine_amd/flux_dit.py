@@ -124,7 +124,7 @@ def ingest_state_dict(state_dict, device, scaled: bool, as_linear=None):
         elif key.endswith(".bias"):
             biases[key[: -len(".bias")]] = t.to(device, torch.bfloat16).contiguous()
         else:
-            other[key] = t.to(device, torch.bfloat16).contiguous()
+            other[key] = (t.to(device, torch.bfloat16) if torch.is_floating_point(t) else t.to(device)).contiguous()
     for name, sc in scales.items():
         if name not in lin:
             raise KeyError("%s%s has no matching weight" % (name, SCALE_SUFFIX))
