@@ -117,13 +117,18 @@ def wan_state_dict_stream(cfg, device, seed=0, std=0.02):
     yield "head.modulation", (torch.randn(1, 2, d, generator=g, device=device) / d ** 0.5).to(bf)
 
 
-def run_wan(args, torch, dev):
+def run_wan(torch, dev, layers, steps, warmup, with_cpu_baseline):
     """BASELINE configs[4]: one Wan2.1-14B DiT denoising step, 21 x 60 x 104 latent = 32 760 tokens, 512 text
-    tokens, 40 layers; every Linear through the scaled e4m3 GEMM."""
+    tokens, `layers` of the 40 layers; every Linear through the scaled e4m3 GEMM.  Returns the result line."""
     from diffsynth_engine_amd.wan_dit import WanDiTRunner
 
+    class _A:
+        pass
+
+    args = _A()
+    args.steps, args.warmup, args.no_cpu_baseline = steps, warmup, not with_cpu_baseline
     cfg = dict(dim=5120, in_dim=16, ffn_dim=13824, out_dim=16, text_dim=4096, freq_dim=256, eps=1e-6,
-               patch_size=(1, 2, 2), num_heads=40, num_layers=args.wan_layers)
+               patch_size=(1, 2, 2), num_heads=40, num_layers=layers)
     runner = WanDiTRunner(wan_state_dict_stream(cfg, dev), cfg, scaled=True, device=dev)
     g = torch.Generator(device=dev).manual_seed(0)
     x = torch.randn(1, 16, 21, 60, 104, generator=g, device=dev).to(torch.bfloat16)
@@ -160,7 +165,7 @@ def run_wan(args, torch, dev):
     gemm = L * (2.0 * S * d * d * 4 + 2.0 * S * d * f * 2 + 2.0 * S * d * d * 2 + 2.0 * 512 * d * d * 2)
     attn = L * (4.0 * S * S * d + 4.0 * S * 512 * d)
     t_ideal = gemm / PEAK_FP8 + attn / PEAK_BF16
-    print(json.dumps({
+    return {
         "metric": "wan2.1_14b_480p_fp8_dit_step_ms", "value": round(ms, 1), "unit": "ms", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 1), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3 GEMM (fp32 accumulate) + bf16 attention",
@@ -178,7 +183,7 @@ def run_wan(args, torch, dev):
                    "attention_in_step": {"ms_per_step": round(attn_secs * 1e3 / args.steps, 1)}},
         "step_roofline": {"algorithmic_tflop": round((gemm + attn) / 1e12, 1), "ideal_ms": round(t_ideal * 1e3, 1),
                           "frac": round(t_ideal * 1e3 / ms, 4)},
-        "cpu_baseline": None if args.no_cpu_baseline else wan_cpu_baseline(cfg, S)}))
+        "cpu_baseline": None if args.no_cpu_baseline else wan_cpu_baseline(cfg, S)}
 
 
 def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
@@ -595,7 +600,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload == "wan14b":
-        return run_wan(args, torch, dev)
+        print(json.dumps(run_wan(torch, dev, args.wan_layers, args.steps, args.warmup, not args.no_cpu_baseline)))
+        return
 
     runner = FluxDiTRunner(flux_state_dict_stream(args.double, args.single, dev), args.double, args.single,
                            scaled=True, device=dev)
@@ -670,6 +676,17 @@ def main():
         result["detail"]["mfma_ceiling_probe"] = mfma_ceiling(torch, dev)
     del runner
     torch.cuda.empty_cache()
+    if not args.no_micro:
+        # BASELINE configs[4] beside the headline figure, at a depth that keeps the default run short: 4 of the 40
+        # layers of the Wan2.1-14B step at its full 32 760 + 512 tokens (every layer is the same work), same code path
+        # as `--workload wan14b`; `ms_per_layer` x 40 is the full step less the embedders and the head
+        w = run_wan(torch, dev, 4, 2, 1, False)
+        result["detail"]["wan14b_4_of_40_layers"] = {
+            "ms_per_step": w["ms_per_step"], "ms_per_layer": round(w["ms_per_step"] / 4, 2),
+            "extrapolated_40_layer_step_ms": round(w["ms_per_step"] * 10, 0),
+            "attention": w["roofline"], "fp8_gemm_in_step": w["detail"]["fp8_gemm_in_step"],
+            "step_roofline_frac": w["step_roofline"]["frac"]}
+        torch.cuda.empty_cache()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.double, args.single)
         result["detail"]["cpu_config_legs"] = cpu_config_legs()
