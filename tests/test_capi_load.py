@@ -246,3 +246,27 @@ def test_gemm_problem_struct_layout_and_qk_epilogue_checks():
     assert lib.dsx_fp8_gemm_grouped(problem(K=144, lda=144, ldw=144), 1, None) == _lib.DSX_EBADSHAPE  # K % 128
     assert lib.dsx_fp8_gemm_grouped(problem(M=8), 1, None) == _lib.DSX_EBADSHAPE               # the GEMV path has none
     assert lib.dsx_fp8_gemm_grouped(problem(rope=p16 + 4), 1, None) == _lib.DSX_EALIGN
+
+
+def test_header_compiles_as_c99_and_agrees_with_the_ctypes_mirrors(tmp_path):
+    """include/dsx.h is a C header (the boundary is a C ABI): it has to compile with a C compiler, and the struct
+    sizes a C caller sees must be the ones the ctypes mirrors use."""
+    import shutil
+    import subprocess
+
+    from diffsynth_engine_amd import _lib
+
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "h.c"
+    src.write_text('#include <stdio.h>\n#include "dsx.h"\nint main(void) { printf("%zu %zu %d %lld\\n", '
+                   'sizeof(dsx_attn_params), sizeof(dsx_gemm_problem), DSX_ABI_VERSION, '
+                   '(long long)DSX_ATTN_STATIC_SCRATCH_BYTES); return 0; }\n')
+    exe = tmp_path / "h"
+    subprocess.run([cc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe)], check=True)
+    attn, gemm, abi, scratch = map(int, subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split())
+    assert attn == ctypes.sizeof(_lib.AttnParams) and gemm == ctypes.sizeof(_lib.GemmProblem)
+    assert abi == _lib.ABI_VERSION == _lib.load().dsx_abi_version()
+    assert scratch == _lib.load().dsx_attn_static_scratch_bytes()
