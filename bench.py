@@ -148,11 +148,23 @@ def run_wan(torch, dev, layers, steps, warmup, with_cpu_baseline):
         n_attn, attn_flops, attn_secs = at.summary()
         n_gemm, gemm_flops, gemm_secs = gt.summary()
     assert torch.isfinite(out.float()).all().item(), "non-finite output"
+    # the same step with the device-side score bound off (every self-attention keeps its running maximum)
+    runner.device_score_bound = False
+    runner(x, ctx, t)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(2):
+        runner(x, ctx, t)
+    torch.cuda.synchronize()
+    ms_scan = (time.perf_counter() - t0) * 1e3 / 2
+    runner.device_score_bound = True
     # sampled-row parity of the timed configuration: the last layer's self-attention shape through the same entry
-    # point against torch's fp32 SDPA on a few query rows of three heads
+    # point (the largest head norms of q and k on the device, as the step's norm kernels leave them) against
+    # torch's fp32 SDPA on a few query rows of three heads
     gq = torch.Generator(device=dev).manual_seed(1)
     q, k, v = [torch.randn(1, 32760, 5120, generator=gq, device=dev, dtype=torch.bfloat16) for _ in range(3)]
-    o = runner._attention(q, k, v).view(1, 32760, 40, 128)
+    n2 = lambda tt: tt.view(32760 * 40, 128).float().square().sum(-1).max()
+    o = runner._attention(q, k, v, torch.stack([n2(q), n2(k)])).view(1, 32760, 40, 128)
     rows = torch.tensor([0, 255, 16383, 32759], device=dev)
     for h in (0, 21, 39):
         hs = lambda tt: tt.view(1, 32760, 40, 128)[:, :, h].float()
@@ -180,7 +192,8 @@ def run_wan(torch, dev, layers, steps, warmup, with_cpu_baseline):
         "detail": {"fp8_gemm_in_step": {"launches": n_gemm, "tflops": round(gemm_flops / gemm_secs / 1e12, 1),
                                         "frac_fp8_peak": round(gemm_flops / gemm_secs / PEAK_FP8, 4),
                                         "ms_per_step": round(gemm_secs * 1e3 / args.steps, 1)},
-                   "attention_in_step": {"ms_per_step": round(attn_secs * 1e3 / args.steps, 1)}},
+                   "attention_in_step": {"ms_per_step": round(attn_secs * 1e3 / args.steps, 1)},
+                   "ms_per_step_without_device_score_bound": round(ms_scan, 1)},
         "step_roofline": {"algorithmic_tflop": round((gemm + attn) / 1e12, 1), "ideal_ms": round(t_ideal * 1e3, 1),
                           "frac": round(t_ideal * 1e3 / ms, 4)},
         "cpu_baseline": None if args.no_cpu_baseline else wan_cpu_baseline(cfg, S)}

@@ -21,7 +21,7 @@ DSX_EARCH = -3
 DSX_ELAUNCH = -4
 DSX_ENULL = -5
 DSX_EWORKSPACE = -6
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class AttnParams(ctypes.Structure):
@@ -49,6 +49,7 @@ class AttnParams(ctypes.Structure):
         ("score_bound", ctypes.c_float),
         ("workspace", c_void_p),
         ("workspace_bytes", c_int64),
+        ("qk_norm2_max", c_void_p),
     ]
 
 
@@ -103,7 +104,7 @@ SIGNATURES = {
     "dsx_rmsnorm_rope_qk": (c_int, [c_void_p, c_int64, c_int64, ctypes.c_int32, ctypes.c_int32, c_void_p, c_void_p,
                                     c_float, c_void_p, c_int64, c_int64, ctypes.c_int32, c_int64, c_void_p]),
     "dsx_rmsnorm_rows": (c_int, [c_void_p, c_int64, c_void_p, c_float, c_void_p, c_int64, c_int64, c_void_p, c_int64,
-                                 c_int64, c_int64, c_void_p]),
+                                 c_int64, c_int64, c_void_p, c_void_p]),
     "dsx_adaln_modulate": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p,
                                    c_float, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64,
                                    c_void_p]),

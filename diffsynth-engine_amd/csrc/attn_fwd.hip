@@ -135,6 +135,11 @@ static int attn_validate(const dsx_attn_params* p) {
     if (((uintptr_t)p->q_norm_w[g] & 15) || ((uintptr_t)p->k_norm_w[g] & 15)) return DSX_EALIGN;
   if (p->workspace && ((uintptr_t)p->workspace & 15)) return DSX_EALIGN;
   if (p->workspace && p->workspace_bytes < 0) return DSX_EBADSHAPE;
+  if (p->qk_norm2_max) {
+    if ((uintptr_t)p->qk_norm2_max & 3) return DSX_EALIGN;
+    // the two maxima describe q and k as given; fused pre-processing would change the rows behind them
+    if (p->rope || p->q_norm_w[0] || p->q_norm_w[1] || p->k_norm_w[0] || p->k_norm_w[1]) return DSX_EBADSHAPE;
+  }
   return DSX_OK;
 }
 

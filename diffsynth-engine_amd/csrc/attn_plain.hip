@@ -64,6 +64,7 @@ __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(
 struct AttnSplit {
   int full_units, tail_units, pieces, len, max_parts;
   float* slots;
+  int device_bound;  // the kernel reads p.qk_norm2_max and returns at once when the other variant is the one to run
 };
 constexpr int kSlotOFloats = QB * HD;               // O part: [dt][rq][wave][g][j][4]
 constexpr int kSlotFloats = kSlotOFloats + 2 * QB;  // + row sums, + references
@@ -95,6 +96,13 @@ __device__ __forceinline__ void store_output(const dsx_attn_params& p, int b, in
 template <bool SCAN, bool SPLIT, bool QPRE>
 __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, AttnSplit sp) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  if (sp.device_bound) {
+    // Both variants were launched; the two device floats say which one works.  Not bounded (Inf and NaN
+    // included, for which the comparison is false) means the variant with the running maximum.
+    const float a = p.qk_norm2_max[0], b = p.qk_norm2_max[1];
+    const bool bounded = sqrtf(a) * sqrtf(b) * p.softmax_scale * (kLog2e * 1.02f) <= kRescaleThreshold;
+    if (bounded == SCAN) return;
+  }
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;  // 0..7
@@ -584,7 +592,7 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   const int64_t Sq = p.sq[0] + p.sq[1], Skv = p.skv[0] + p.skv[1];
   const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
   const int nkb = (int)((Skv + KB - 1) / KB);
-  sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr};
+  sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr, 0};
   if (p.rope || p.q_norm_w[0] || p.q_norm_w[1]) return 0;  // the split kernel has no q pre-processing
   if (cus <= 0) return 0;                                    // no device to ask
   const int tail = (int)(units % cus);
@@ -643,7 +651,7 @@ int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_b
   AttnSplit sp;
   const int64_t need = plan_split(p, device_cus(), sp);
   if (need == 0 || !scratch || scratch_bytes < need || ((uintptr_t)scratch & 15))
-    sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr};
+    sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr, 0};
   else
     sp.slots = (float*)scratch;
   dim3 grid((unsigned)(((sp.full_units + 7) / 8) * 8 + sp.pieces)), block(512);
@@ -652,7 +660,18 @@ int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_b
   const bool bounded = p.score_bound > 0.f && p.score_bound * kLog2e <= kRescaleThreshold;
   const bool split = sp.tail_units > 0;
   const bool qpre = p.rope || p.q_norm_w[0] || p.q_norm_w[1];  // (never together with the split)
-  if (qpre && bounded)
+  sp.device_bound = 0;
+  if (p.qk_norm2_max && !bounded && !qpre) {
+    // the bound lives on the device: launch both variants, each looks at it and one of them returns at once
+    sp.device_bound = 1;
+    if (split) {
+      attn_plain_kernel<false, true, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+      attn_plain_kernel<true, true, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+    } else {
+      attn_plain_kernel<false, false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+      attn_plain_kernel<true, false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
+    }
+  } else if (qpre && bounded)
     attn_plain_kernel<false, false, true><<<grid, block, kLdsBytes, st>>>(p, sp);
   else if (qpre)
     attn_plain_kernel<true, false, true><<<grid, block, kLdsBytes, st>>>(p, sp);

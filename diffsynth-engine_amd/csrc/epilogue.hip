@@ -213,7 +213,8 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const uint16_t* __res
                                                            const uint16_t* __restrict__ w, float eps,
                                                            const float* __restrict__ rope, int64_t rope_sb,
                                                            int64_t rows_per_batch, uint16_t* __restrict__ out,
-                                                           int64_t ldo, int64_t rows, int D) {
+                                                           int64_t ldo, int64_t rows, int D,
+                                                           float* head_norm2_max) {
   __shared__ float red[4];
   const int t = threadIdx.x % TPR;
   int64_t row = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
@@ -245,29 +246,59 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const uint16_t* __res
     ss += ok[i] ? part : 0.f;
   }
   const float rrms = rsqrtf(row_sum<TPR>(ss, red) / (float)D + eps);
-  if (!live) return;  // wave-uniform
-  const float* rp = rope ? rope + (row / rows_per_batch) * rope_sb + (row % rows_per_batch) * 128 : nullptr;
+  float hmax = 0.f;
+  if (live) {  // wave-uniform
+    const float* rp = rope ? rope + (row / rows_per_batch) * rope_sb + (row % rows_per_batch) * 128 : nullptr;
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    float wv[8];
-    unpack8(wraw[i], wv);
-    float v[8];
+    for (int i = 0; i < NCH; ++i) {
+      float wv[8];
+      unpack8(wraw[i], wv);
+      float v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = round_bf16(round_bf16(val[i][j] * rrms) * wv[j]);
-    if (rp) {
-      const int off = (cc[i] * 8) & 127;  // offset inside the head: floats (cos, sin) of pairs off/2 .. off/2+3
-      const f32x4 t0 = *reinterpret_cast<const f32x4*>(rp + off);
-      const f32x4 t1 = *reinterpret_cast<const f32x4*>(rp + off + 4);
-      const float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+      for (int j = 0; j < 8; ++j) v[j] = round_bf16(round_bf16(val[i][j] * rrms) * wv[j]);
+      if (rp) {
+        const int off = (cc[i] * 8) & 127;  // offset inside the head: floats (cos, sin) of pairs off/2 .. off/2+3
+        const f32x4 t0 = *reinterpret_cast<const f32x4*>(rp + off);
+        const f32x4 t1 = *reinterpret_cast<const f32x4*>(rp + off + 4);
+        const float cs[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const float co = cs[2 * k], sn = cs[2 * k + 1];
-        const float x0 = v[2 * k], x1 = v[2 * k + 1];
-        v[2 * k] = mul_add_unfused(co, x0, -sn, x1);
-        v[2 * k + 1] = mul_add_unfused(sn, x0, co, x1);
+        for (int k = 0; k < 4; ++k) {
+          const float co = cs[2 * k], sn = cs[2 * k + 1];
+          const float x0 = v[2 * k], x1 = v[2 * k + 1];
+          v[2 * k] = mul_add_unfused(co, x0, -sn, x1);
+          v[2 * k + 1] = mul_add_unfused(sn, x0, co, x1);
+        }
+      }
+      if (ok[i]) reinterpret_cast<u32x4*>(out + row * ldo)[cc[i]] = pack8(v);
+      if (head_norm2_max) {  // uniform
+        // a 128-wide head is 16 chunks = the 16 lanes of one DPP row (TPR is a multiple of 16)
+        float n2 = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) n2 += v[j] * v[j];
+        n2 = ok[i] ? n2 : 0.f;
+        n2 += dpp_f32<kDppRowRor8>(n2);
+        n2 += dpp_f32<kDppRowRor4>(n2);
+        n2 += dpp_f32<kDppQuadXor2>(n2);
+        n2 += dpp_f32<kDppQuadXor1>(n2);
+        hmax = fmaxf(hmax, n2);
       }
     }
-    if (ok[i]) reinterpret_cast<u32x4*>(out + row * ldo)[cc[i]] = pack8(v);
+  }
+  if (head_norm2_max) {
+    // One look at the current maximum per workgroup, one atomic only when it has to rise.  The look is a
+    // device-scope load (the eight L2s do not see each other's atomics otherwise) and the value only ever
+    // grows, so a stale look costs one redundant atomic and nothing else.  Non-negative floats order like
+    // their bit patterns; +Inf stays the maximum once seen.
+    hmax = wave_max(hmax);
+    const int w = threadIdx.x >> 6;
+    __syncthreads();  // `red` may still be read by the row sum of a slower wave
+    if ((threadIdx.x & 63) == 0) red[w] = hmax;
+    __syncthreads();
+    if (threadIdx.x == 0) {  // (waves of rows past the end bring 0)
+      hmax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+      const float seen = __hip_atomic_load(head_norm2_max, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (!(hmax <= seen)) atomicMax(reinterpret_cast<unsigned int*>(head_norm2_max), __float_as_uint(hmax));
+    }
   }
 }
 
@@ -483,22 +514,21 @@ extern "C" int dsx_flow_match_euler_step(const void* latents, const void* v, flo
 
 extern "C" int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float eps, const float* rope,
                                 int64_t rope_sb, int64_t rows_per_batch, void* out, int64_t ldo, int64_t rows,
-                                int64_t D, void* stream) {
+                                int64_t D, float* head_norm2_max, void* stream) {
   using namespace dsx;
   if (rows == 0) return DSX_OK;
   if (!x || !w || !out) return DSX_ENULL;
   if (rows < 0 || D <= 0 || (D & 7) || D > 16384 || ldx < D || ldo < D || rows_per_batch <= 0 ||
-      (rope && (D & 127)))
+      ((rope || head_norm2_max) && (D & 127)))
     return DSX_EBADSHAPE;
   if ((ldx & 7) || (ldo & 7) || (rope_sb & 3) || misaligned16(x) || misaligned16(out) || misaligned16(w) ||
-      misaligned16(rope))
+      misaligned16(rope) || ((uintptr_t)head_norm2_max & 3))
     return DSX_EALIGN;
-  if (rows == 0) return DSX_OK;
   hipStream_t st = (hipStream_t)stream;
 #define DSX_LAUNCH_RMS(NCH, TPR)                                                                           \
   rmsnorm_rows_kernel<NCH, TPR><<<dim3((unsigned)((rows + 256 / TPR - 1) / (256 / TPR))), dim3(256), 0, st>>>( \
       (const uint16_t*)x, ldx, (const uint16_t*)w, eps, rope, rope_sb, rows_per_batch, (uint16_t*)out, ldo,   \
-      rows, (int)D)
+      rows, (int)D, head_norm2_max)
   if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_RMS(6, 64);
   else if (D > 4096 && D <= 1024 * 5 && rows >= 2048) DSX_LAUNCH_RMS(5, 128);  // as for AdaLN
   else if (D <= 2048 * 3) DSX_LAUNCH_RMS(3, 256);

@@ -218,7 +218,7 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
                    rope: Optional[torch.Tensor] = None, q_norm_w=None, k_norm_w=None, q2_norm_w=None,
                    k2_norm_w=None, eps: float = 1e-6, out: Optional[torch.Tensor] = None,
                    out2: Optional[torch.Tensor] = None, score_bound: float = 0.0, split_keys: bool = True,
-                   static_scratch: bool = False):
+                   static_scratch: bool = False, qk_norm2_max: Optional[torch.Tensor] = None):
     """softmax(q k^T * scale) v over the concatenation [segment 1, segment 2] of rows.
 
     q, k, v: (B,H,S,128) bf16 views with unit stride in the last dim (any other strides).
@@ -234,6 +234,9 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     than it holds raises.
     score_bound: optional promise |scale * q.k| <= score_bound for every pair (after RMSNorm/RoPE); when it is
     small enough the kernel skips the running softmax maximum (same result).  0 = no promise.
+    qk_norm2_max: optional fp32 device tensor of two values, upper bounds of |q row|^2 and |k row|^2 over every
+    head row the call reads (rmsnorm_rows(..., head_norm2_max=) leaves them); the kernels read it on the device
+    and skip the running maximum when the bound it implies is small enough.  Not with rope / *_norm_w.
     Returns out (B,H,Sq1,128)-shaped view semantics: writes `out` (B,Sq1,H,128 layout allowed via strides).
     """
     _require_cuda(q, k, v)
@@ -282,6 +285,12 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
                 getattr(P, name)[i] = _ptr(w)
     P.norm_eps = eps
     P.score_bound = float(score_bound)
+    if qk_norm2_max is not None:
+        if qk_norm2_max.dtype != torch.float32 or qk_norm2_max.numel() != 2 or not qk_norm2_max.is_contiguous() \
+                or qk_norm2_max.device != q.device:
+            raise ValueError("qk_norm2_max must be two contiguous fp32 values on the device of q")
+        keep.append(qk_norm2_max)
+        P.qk_norm2_max = _ptr(qk_norm2_max)
     lib = _lib.load()
     # scratch for the one-off k pre-pass and for splitting the key range of a partly filled last round
     if static_scratch:
@@ -344,9 +353,11 @@ def rmsnorm_rope_qk(qkv: torch.Tensor, heads_q: int, heads_k: int, q_norm_w: Opt
 
 
 def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, rope: Optional[torch.Tensor] = None,
-                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 out: Optional[torch.Tensor] = None, head_norm2_max: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Wan-style RMSNorm over the full last dim of (B,S,D) (or (rows,D)) bf16, optionally followed by RoPE on
-    every 128-wide head with the fp32 (B|1, S, 64, 2) (cos, sin) table."""
+    every 128-wide head with the fp32 (B|1, S, 64, 2) (cos, sin) table.
+    head_norm2_max: optional one-element fp32 device tensor, raised to the largest squared 2-norm of a 128-wide
+    head of an output row (never lowered: zero it before the first contributing call)."""
     _require_cuda(x)
     if x.dtype != _BF16:
         raise ValueError("rmsnorm_rows expects bf16")
@@ -367,8 +378,11 @@ def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, rope:
     else:
         o2, ldo = _rows_2d(out)
     w = weight.to(_BF16).contiguous()
+    if head_norm2_max is not None and (head_norm2_max.dtype != torch.float32 or head_norm2_max.numel() != 1
+                                       or head_norm2_max.device != x.device):
+        raise ValueError("head_norm2_max must be one fp32 value on the device of x")
     rc = _lib.load().dsx_rmsnorm_rows(_ptr(x2), ldx, _ptr(w), eps, _ptr(rope), rope_sb, rows_per_batch, _ptr(o2), ldo,
-                                      rows, D, _stream())
+                                      rows, D, _ptr(head_norm2_max), _stream())
     _lib.check(rc, "dsx_rmsnorm_rows")
     return out.view(shp)
 

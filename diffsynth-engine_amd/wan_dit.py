@@ -26,6 +26,9 @@ class WanDiTRunner:
         self.cfg = cfg
         self.device = torch.device(device)
         self.scaled = scaled
+        # self-attention reads the largest head norms of q and k on the device and drops the running softmax
+        # maximum when they allow it (False: always the running maximum)
+        self.device_score_bound = True
         d = cfg["dim"]
 
         def conv_as_linear(key, t):  # Conv3d with kernel == stride is a Linear over each patch
@@ -67,14 +70,15 @@ class WanDiTRunner:
                          aw.view(1, 1, w, -1).expand(f, h, w, -1)], dim=-1).reshape(1, f * h * w, -1)
         return torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).float().contiguous()
 
-    def _attention(self, q, k, v):
-        """(B,S,H*D) projections -> (B,S,H*D) attention output, head split/merge by strides (wan_dit.py:18-22)."""
+    def _attention(self, q, k, v, qk_norm2_max=None):
+        """(B,S,H*D) projections -> (B,S,H*D) attention output, head split/merge by strides (wan_dit.py:18-22).
+        qk_norm2_max: the largest squared head norms of q and k, on the device (see ops.attention_bhsd)."""
         H = self.cfg["num_heads"]
         B, Sq, HD = q.shape
         D = HD // H
         sp = lambda t: t.view(t.shape[0], t.shape[1], H, D).transpose(1, 2)
         out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=q.device)
-        ops.attention_bhsd(sp(q), sp(k), sp(v), out=out.transpose(1, 2))
+        ops.attention_bhsd(sp(q), sp(k), sp(v), out=out.transpose(1, 2), qk_norm2_max=qk_norm2_max)
         return out.view(B * Sq, HD)
 
     # ------------------------------------------------------------------ block
@@ -89,10 +93,16 @@ class WanDiTRunner:
         # self-attention
         hq, hs = self._modulate_q(x, m[1], m[0])
         hq = hq.view(B * S, d)
-        q = ops.rmsnorm_rows(L[p + "self_attn.q"](hq, hs).view(B, S, d), V[p + "self_attn.norm_q.weight"], eps, rope)
-        k = ops.rmsnorm_rows(L[p + "self_attn.k"](hq, hs).view(B, S, d), V[p + "self_attn.norm_k.weight"], eps, rope)
+        # The RMSNorm runs over all heads at once, so no static bound on a head's scores exists; the norm kernels
+        # leave the largest squared head norm of q and of k on the device and the attention kernels read it there
+        # (|q.k| <= |q||k|): with ordinary activations the running softmax maximum is not needed.
+        nm = torch.zeros(2, dtype=torch.float32, device=x.device) if self.device_score_bound else None
+        q = ops.rmsnorm_rows(L[p + "self_attn.q"](hq, hs).view(B, S, d), V[p + "self_attn.norm_q.weight"], eps, rope,
+                             head_norm2_max=None if nm is None else nm[0:1])
+        k = ops.rmsnorm_rows(L[p + "self_attn.k"](hq, hs).view(B, S, d), V[p + "self_attn.norm_k.weight"], eps, rope,
+                             head_norm2_max=None if nm is None else nm[1:2])
         v = L[p + "self_attn.v"](hq, hs).view(B, S, d)
-        aq, asc = self._q(self._attention(q, k, v))
+        aq, asc = self._q(self._attention(q, k, v, nm))
         x2 = L[p + "self_attn.o"](aq, asc, resid=x2, gate=m[2], rows_per_batch=S)
         # cross-attention (no gate on the residual)
         hq, hs = self._modulate_q(x2.view(B, S, d), None, None, V[p + "norm3.weight"], V[p + "norm3.bias"])

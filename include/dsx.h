@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define DSX_ABI_VERSION 4
+#define DSX_ABI_VERSION 5
 
 enum {
   DSX_OK = 0,
@@ -208,6 +208,16 @@ typedef struct dsx_attn_params {
    * Calls that share a scratch must not overlap. */
   void* workspace;
   int64_t workspace_bytes;
+  /* Optional score bound read ON THE DEVICE when the kernels run (NULL = none): two floats,
+   * [0] >= |q row|^2 and [1] >= |k row|^2 (squared 2-norms over head_dim) for every (batch, head, row) the call
+   * reads, e.g. the maxima dsx_rmsnorm_rows leaves in its head_norm2_max.  |q.k| <= sqrt([0]*[1]) bounds every
+   * score; when softmax_scale*log2(e)*sqrt([0]*[1]) (plus 1 % for roundings) is at most 64 the kernel that keeps
+   * the softmax reference at 0 does the work, otherwise (Inf and NaN included) the one with the running maximum
+   * does: both are launched and the one not chosen returns at once, so the host never waits for the values and
+   * the call can sit in a captured graph.  Same softmax either way.  Not combined with the fused pre-processing
+   * (rope, *_norm_w change the rows the bound describes): DSX_EBADSHAPE.  Ignored when score_bound already
+   * holds a promise.  Unlike score_bound this one cannot be wrong as long as the two floats are true maxima. */
+  const float* qk_norm2_max;
 } dsx_attn_params;
 
 int dsx_attn_fwd(const dsx_attn_params* p, void* stream);
@@ -266,9 +276,13 @@ int dsx_rmsnorm_rope_qk(void* x, int64_t x_sb, int64_t x_ss, int32_t heads_q, in
  * Replaces Wan's RMSNorm.forward over the full model dim (models/wan/wan_dit.py:61-78,98-99,142-143) and
  * rope_apply (wan_dit.py:54-58; the reference multiplies in complex128, this kernel in fp32).
  * x, out: (rows, D) bf16; w: (D,) bf16; rope: fp32 (pos, 64, 2) or NULL.  D % 8 == 0 (128 with rope), D <= 16384.
+ * head_norm2_max (device, one float, or NULL; needs D % 128 == 0): raised (atomic maximum, never lowered) to the
+ * largest squared 2-norm of a 128-wide head of an output row; the caller sets it to 0 before the first call
+ * that contributes.  It is what dsx_attn_params.qk_norm2_max reads (no counterpart in the reference).
  */
 int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float eps, const float* rope, int64_t rope_sb,
-                     int64_t rows_per_batch, void* out, int64_t ldo, int64_t rows, int64_t D, void* stream);
+                     int64_t rows_per_batch, void* out, int64_t ldo, int64_t rows, int64_t D, float* head_norm2_max,
+                     void* stream);
 
 /*
  * AdaLN modulate: y = LayerNorm(x; eps, no affine) * (1 + scale) + shift, one row per token.

@@ -32,7 +32,7 @@ def test_abi_version_and_strerror():
     from diffsynth_engine_amd import _lib
 
     lib = _lib.load()
-    assert lib.dsx_abi_version() == 4
+    assert lib.dsx_abi_version() == 5
     assert _lib.strerror(0) == "ok"
     for code in (-1, -2, -3, -4, -5, -6):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
@@ -44,7 +44,7 @@ def test_attn_params_struct_layout_matches_header():
 
     # q,k,v,o,sq,skv = 6*16; 12 stride pairs * 16; 3 int32 + float; rope, rope_sb, rope_rows;
     # 2*16 norm pointers; two floats; workspace pointer + byte count
-    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 8 + 32 + 8 + 16
+    assert ctypes.sizeof(_lib.AttnParams) == 6 * 16 + 12 * 16 + 16 + 8 + 8 + 8 + 32 + 8 + 16 + 8
 
 
 def test_null_and_shape_errors_without_touching_the_gpu():

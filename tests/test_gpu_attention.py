@@ -266,3 +266,50 @@ def test_q_only_rmsnorm_needs_no_scratch(dev):
     assert _lib.load().dsx_attn_workspace_bytes(P) == 0
     got = ops.attention_bhsd(q.to(dev), k.to(dev), v.to(dev), q_norm_w=wd).cpu()
     assert _rel_err(got, want) <= TOL
+
+
+@pytest.mark.parametrize("H,Sq,Skv", [(4, 520, 777), (3, 2048, 2100)])  # whole units; the key-range split
+def test_device_side_score_bound_picks_the_kernel(dev, H, Sq, Skv):
+    """qk_norm2_max: the two device floats choose between the kernel with a fixed softmax reference and the one
+    with the running maximum without the host ever reading them.  Small norms give bit for bit the output of a
+    host-side promise (score_bound), large or non-finite ones the output of the default path; the result is the
+    same softmax either way."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(H + Sq)
+    q, k, v = [torch.randn(1, H, s, 128, generator=g).bfloat16().to(dev) for s in (Sq, Skv, Skv)]
+    n2 = lambda t: t.float().square().sum(-1).max()
+    scale = 128 ** -0.5
+
+    def bound_of(a, b):
+        return float((n2(a) * n2(b)).sqrt()) * scale
+
+    # N(0,1) rows: |q||k| * scale ~ 128 / 11.3 -> log2 domain ~ 18: bounded
+    nm = torch.stack([n2(q), n2(k)])
+    assert bound_of(q, k) * 1.4427 * 1.02 < 64
+    promised = ops.attention_bhsd(q, k, v, score_bound=bound_of(q, k))
+    default = ops.attention_bhsd(q, k, v)
+    assert torch.equal(ops.attention_bhsd(q, k, v, qk_norm2_max=nm), promised)
+    assert _rel_err(promised.cpu(), O.sdpa(q.float().cpu(), k.float().cpu(), v.float().cpu())) <= TOL
+    # the same rows, but a bound that does not allow it (true for q * 12; here deliberately pessimistic), Inf, NaN
+    for bad in (torch.stack([n2(q) * 144, n2(k)]), torch.tensor([float("inf"), 1.0], device=dev),
+                torch.tensor([1.0, float("nan")], device=dev)):
+        assert torch.equal(ops.attention_bhsd(q, k, v, qk_norm2_max=bad), default)
+    # rows that need the running maximum, with their true norms
+    q12 = (q.float() * 12).bfloat16()
+    nm12 = torch.stack([n2(q12), n2(k)])
+    assert bound_of(q12, k) * 1.4427 > 64
+    assert torch.equal(ops.attention_bhsd(q12, k, v, qk_norm2_max=nm12), ops.attention_bhsd(q12, k, v))
+    # a host-side promise wins over the device floats
+    assert torch.equal(ops.attention_bhsd(q, k, v, score_bound=bound_of(q, k), qk_norm2_max=bad), promised)
+
+
+def test_device_side_score_bound_not_with_fused_preprocessing(dev):
+    from diffsynth_engine_amd import ops
+
+    q, k, v = [torch.randn(1, 2, 64, 128).bfloat16().to(dev) for _ in range(3)]
+    w = torch.ones(128).bfloat16().to(dev)
+    with pytest.raises(ValueError):
+        ops.attention_bhsd(q, k, v, q_norm_w=w, qk_norm2_max=torch.ones(2, device=dev))
+    with pytest.raises(ValueError):
+        ops.attention_bhsd(q, k, v, qk_norm2_max=torch.ones(3, device=dev))

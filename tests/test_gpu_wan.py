@@ -97,3 +97,39 @@ def test_two_layers_at_the_14b_width(dev):
     assert got.shape == want.shape
     c, floor = _cos(got, want), _cos(want, want_nudged)
     assert c >= 0.99 and c >= min(0.999, floor - 1e-3), (c, floor)
+
+
+@pytest.mark.parametrize("S,D", [(24, 256), (1100, 1536), (700, 3072), (2049, 5120), (33, 8192)])
+def test_rmsnorm_rows_leaves_the_largest_squared_head_norm(dev, S, D):
+    """head_norm2_max: every launch shape of the row kernel (64, 128 and 256 lanes per row) raises the float to
+    max over (row, head) of |y_head|^2 of the rows it wrote; it is never lowered."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(D + S)
+    x = (torch.randn(1, S, D, generator=g) * 2).bfloat16()
+    x[0, S // 3, 128:256] *= 5  # one head of one row stands out
+    w = (1 + 0.1 * torch.randn(D, generator=g)).bfloat16()
+    fr = ow.freqs_cis_3d(128, 1, 1, S)
+    table = torch.stack((fr.real, fr.imag), dim=-1).float().reshape(1, S, 64, 2).to(dev)
+    for rope in (None, table):
+        nm = torch.zeros(1, dtype=torch.float32, device=dev)
+        y = ops.rmsnorm_rows(x.to(dev), w.to(dev), 1e-6, rope, head_norm2_max=nm)
+        assert torch.equal(y, ops.rmsnorm_rows(x.to(dev), w.to(dev), 1e-6, rope))  # the rows themselves are unchanged
+        want = y.float().view(S, D // 128, 128).square().sum(-1)
+        assert int(want.argmax()) == (S // 3) * (D // 128) + 1
+        # the kernel sums the fp32 values before their bf16 rounding: 2^-8 relative on a squared norm
+        assert abs(nm.item() - want.max().item()) <= 2 ** -7 * want.max().item()
+        big = torch.full((1,), 1e9, dtype=torch.float32, device=dev)
+        ops.rmsnorm_rows(x.to(dev), w.to(dev), 1e-6, rope, head_norm2_max=big)
+        assert big.item() == 1e9
+    with pytest.raises(ValueError):
+        ops.rmsnorm_rows(x.to(dev), w.to(dev), 1e-6, head_norm2_max=torch.zeros(2, device=dev))
+
+
+def test_rmsnorm_rows_head_norm_needs_whole_heads(dev):
+    from diffsynth_engine_amd import _lib, ops
+
+    x = torch.randn(4, 192).bfloat16().to(dev)
+    with pytest.raises(ValueError) as e:
+        ops.rmsnorm_rows(x, torch.ones(192).bfloat16().to(dev), head_norm2_max=torch.zeros(1, device=dev))
+    assert "dsx error %d" % _lib.DSX_EBADSHAPE in str(e.value)

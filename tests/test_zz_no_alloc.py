@@ -56,10 +56,15 @@ def _both(dev, H, S, fused, seed):
     P.workspace, P.workspace_bytes = ws.data_ptr(), need
     assert lib.dsx_attn_fwd(P, stream) == 0
     Ps = _params(_lib, q, k, v, o_static, rope, wq, wk)
-    before = torch.cuda.memory_allocated(dev)
+    # nothing is allocated during the call: neither through torch (its cumulative allocation counter stands still;
+    # the bytes in use may only fall, when the collector frees an earlier test's garbage) nor behind its back
+    # (the device's free memory does not shrink)
+    torch.cuda.synchronize()
+    count = lambda: torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+    before, free_before = count(), torch.cuda.mem_get_info(dev)[0]
     assert lib.dsx_attn_fwd_static(Ps, stream) == 0
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(dev) == before
+    assert count() == before and torch.cuda.mem_get_info(dev)[0] >= free_before
     return o_static, o_ws
 
 
