@@ -109,11 +109,18 @@ def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, res
     elif out.dtype != _BF16 or out.shape != (M, N) or out.stride(1) != 1:
         raise ValueError("fp8_gemm: bad `out`")
     if bias is not None:
+        if bias.numel() != N:
+            raise ValueError("fp8_gemm: bias has %d entries for N = %d" % (bias.numel(), N))
         if bias.dtype != _BF16:
             bias = bias.to(_BF16)
         bias = bias.contiguous()
     if a_scale is not None:
+        if a_scale.dtype != torch.float32 or a_scale.numel() != M:
+            raise ValueError("fp8_gemm: a_scale must hold one fp32 value per row of a")
         a_scale = a_scale.contiguous()
+    if w_scale is not None and (w_scale.dtype != torch.float32 or w_scale.numel() != 1):
+        raise ValueError("fp8_gemm: w_scale must be one fp32 value")
+    _require_cuda(a_scale, w_scale, bias, out, resid, gate)
     gate_sb = 0
     if resid is not None:
         if resid.dtype != _BF16 or resid.shape != (M, N) or resid.stride(1) != 1:
@@ -122,6 +129,9 @@ def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, res
             gate = gate.reshape(-1, N)
             if gate.dtype != _BF16 or gate.stride(1) != 1:
                 gate = gate.to(_BF16).contiguous()
+            rpb = rows_per_batch or max(M, 1)
+            if gate.shape[0] > 1 and gate.shape[0] * rpb < M:
+                raise ValueError("fp8_gemm: %d gate rows of %d tokens do not cover M = %d" % (gate.shape[0], rpb, M))
             gate_sb = gate.stride(0) if gate.shape[0] > 1 else 0
     elif gate is not None:
         raise ValueError("fp8_gemm: `gate` needs `resid`")
@@ -136,6 +146,8 @@ def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, res
         wq, wk, rope = qk.get("q_norm_w"), qk.get("k_norm_w"), qk.get("rope")
         wq = None if wq is None else wq.to(_BF16).contiguous()
         wk = None if wk is None else wk.to(_BF16).contiguous()
+        if any(w is not None and w.numel() != 128 for w in (wq, wk)):
+            raise ValueError("fp8_gemm: q/k RMSNorm weights have 128 entries")
         prob.q_norm_w, prob.k_norm_w = _ptr(wq), _ptr(wk)
         prob.qk_heads, prob.norm_eps = int(qk["heads"]), float(qk.get("eps", 1e-6))
         if rope is not None:
@@ -191,9 +203,23 @@ def fp8_gemm_grouped(problems):
 def fp8_gemv_rowscale(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor],
                       w_row_scale: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Small-M (<= 8) product against a stack of Linear weights with one fp32 weight scale per output row."""
-    _require_cuda(a_q, w_q)
+    _require_cuda(a_q, w_q, a_scale, w_row_scale, bias)
+    if a_q.dtype != FP8 or w_q.dtype != FP8 or a_q.dim() != 2 or w_q.dim() != 2 or a_q.shape[1] != w_q.shape[1]:
+        raise ValueError("fp8_gemv_rowscale expects e4m3 a (M,K) and w (N,K)")
+    if a_q.stride(1) != 1:
+        a_q = a_q.contiguous()
+    if w_q.stride(1) != 1:
+        w_q = w_q.contiguous()
     M, K = a_q.shape
     N = w_q.shape[0]
+    if w_row_scale.dtype != torch.float32 or w_row_scale.numel() != N or not w_row_scale.is_contiguous():
+        raise ValueError("fp8_gemv_rowscale: w_row_scale must hold one contiguous fp32 value per row of w")
+    if a_scale is not None and (a_scale.dtype != torch.float32 or a_scale.numel() != M or not a_scale.is_contiguous()):
+        raise ValueError("fp8_gemv_rowscale: a_scale must hold one contiguous fp32 value per row of a")
+    if bias is not None:
+        if bias.numel() != N:
+            raise ValueError("fp8_gemv_rowscale: bias has %d entries for N = %d" % (bias.numel(), N))
+        bias = bias.to(_BF16).contiguous()
     out = torch.empty((M, N), dtype=_BF16, device=a_q.device)
     rc = _lib.load().dsx_fp8_gemv_rowscale(_ptr(a_q), a_q.stride(0), _ptr(w_q), w_q.stride(0), _ptr(a_scale),
                                            _ptr(w_row_scale), _ptr(bias), _ptr(out), N, M, N, K, _stream())
@@ -246,6 +272,17 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     B, H, S1, D = q.shape
     if D != 128:
         raise ValueError("head_dim must be 128, got %d" % D)
+    if k.shape != v.shape or k.shape[:2] != (B, H) or k.shape[3] != D:
+        raise ValueError("attention: q %s, k %s, v %s do not fit" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
+    if (k2 is None) != (v2 is None) or (k2 is not None and (k2.shape != v2.shape or k2.shape[:2] != (B, H)
+                                                            or k2.shape[3] != D)):
+        raise ValueError("attention: the second key/value segment does not fit the first")
+    if q2 is not None and (q2.shape[:2] != (B, H) or q2.shape[3] != D):
+        raise ValueError("attention: the second query segment does not fit the first")
+    for t, s_ in ((out, S1), (out2, None if q2 is None else q2.shape[2])):
+        if t is not None and (t.dtype != _BF16 or tuple(t.shape) != (B, H, s_, D)):
+            raise ValueError("attention: `out` must be bf16 (B,H,Sq,128)")
+    _require_cuda(q2, k2, v2, out, out2, rope, qk_norm2_max)
     P = _lib.AttnParams()
     S2 = 0 if q2 is None else q2.shape[2]
     Skv1 = k.shape[2]
@@ -270,7 +307,8 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     P.softmax_scale = float(scale) if scale is not None else 1.0 / math.sqrt(D)
     keep = []
     if rope is not None:
-        if rope.dtype != torch.float32 or rope.dim() != 4 or rope.shape[1:] != (S1 + S2, 64, 2):
+        if rope.dtype != torch.float32 or rope.dim() != 4 or rope.shape[1:] != (S1 + S2, 64, 2) \
+                or rope.shape[0] not in (1, B):
             raise ValueError("rope table must be fp32 (B|1, Sq, 64, 2)")
         rope = rope.contiguous()
         keep.append(rope)
@@ -280,6 +318,8 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     for i, (qw, kw) in enumerate(((q_norm_w, k_norm_w), (q2_norm_w, k2_norm_w))):
         for name, w in (("q_norm_w", qw), ("k_norm_w", kw)):
             if w is not None:
+                if w.numel() != D:
+                    raise ValueError("attention: RMSNorm weights have %d entries" % D)
                 w = w.to(_BF16).contiguous()
                 keep.append(w)
                 getattr(P, name)[i] = _ptr(w)
@@ -307,6 +347,16 @@ def attention_bhsd(q, k, v, *, q2=None, k2=None, v2=None, scale: Optional[float]
     return (out, out2) if q2 is not None else out
 
 
+def _rope_table(rope: torch.Tensor, batch: int, rows: int) -> torch.Tensor:
+    """A (B|1, >= rows, 64, 2) fp32 (cos, sin) table on the device, contiguous; the kernels read `rows` rows of it per
+    batch entry and cannot see where it ends."""
+    _require_cuda(rope)
+    if rope.dtype != torch.float32 or rope.dim() != 4 or rope.shape[2:] != (64, 2) or rope.shape[0] not in (1, batch) \
+            or rope.shape[1] < rows:
+        raise ValueError("rope table must be fp32 (B|1, >= %d, 64, 2), got %s" % (rows, tuple(rope.shape)))
+    return rope.contiguous()
+
+
 def rmsnorm_rope(x: torch.Tensor, norm_w: Optional[torch.Tensor], rope: Optional[torch.Tensor], pos0: int = 0,
                  eps: float = 1e-6, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """RMSNorm (per head, 128) then RoPE of a (B,H,S,128) bf16 view; returns a dense (B,H,S,128) tensor."""
@@ -316,11 +366,15 @@ def rmsnorm_rope(x: torch.Tensor, norm_w: Optional[torch.Tensor], rope: Optional
         raise ValueError("rmsnorm_rope expects bf16 (B,H,S,128)")
     if out is None:
         out = torch.empty((B, H, S, D), dtype=_BF16, device=x.device)
+    elif out.dtype != _BF16 or out.shape != x.shape:
+        raise ValueError("rmsnorm_rope: `out` must match x")
     if norm_w is not None:
+        if norm_w.numel() != D:
+            raise ValueError("rmsnorm_rope: the RMSNorm weight has %d entries" % D)
         norm_w = norm_w.to(_BF16).contiguous()
     rope_sb = 0
     if rope is not None:
-        rope = rope.contiguous()
+        rope = _rope_table(rope, B, pos0 + S)
         rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
     xs, os_ = _bhsd_strides(x), _bhsd_strides(out)
     rc = _lib.load().dsx_rmsnorm_rope(_ptr(x), xs[0], xs[1], xs[2], _ptr(norm_w), eps, _ptr(rope), rope_sb, pos0,
@@ -338,13 +392,15 @@ def rmsnorm_rope_qk(qkv: torch.Tensor, heads_q: int, heads_k: int, q_norm_w: Opt
     if qkv.dim() != 3 or qkv.dtype != _BF16 or qkv.stride(2) != 1 or qkv.shape[2] < (heads_q + heads_k) * 128:
         raise ValueError("rmsnorm_rope_qk expects bf16 (B, S, >= (heads_q+heads_k)*128) with unit column stride")
     B, S, _ = qkv.shape
+    if any(w is not None and w.numel() != 128 for w in (q_norm_w, k_norm_w)):
+        raise ValueError("rmsnorm_rope_qk: RMSNorm weights have 128 entries")
     if q_norm_w is not None:
         q_norm_w = q_norm_w.to(_BF16).contiguous()
     if k_norm_w is not None:
         k_norm_w = k_norm_w.to(_BF16).contiguous()
     rope_sb = 0
     if rope is not None:
-        rope = rope.contiguous()
+        rope = _rope_table(rope, B, pos0 + S)
         rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
     rc = _lib.load().dsx_rmsnorm_rope_qk(_ptr(qkv), qkv.stride(0), qkv.stride(1), heads_q, heads_k, _ptr(q_norm_w),
                                          _ptr(k_norm_w), eps, _ptr(rope), rope_sb, pos0, B, S, _stream())
@@ -377,7 +433,10 @@ def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, rope:
         o2, ldo = out, D
     else:
         o2, ldo = _rows_2d(out)
+    if weight.numel() != D:
+        raise ValueError("rmsnorm_rows: the weight has %d entries for D = %d" % (weight.numel(), D))
     w = weight.to(_BF16).contiguous()
+    _require_cuda(w, rope, out)
     if head_norm2_max is not None and (head_norm2_max.dtype != torch.float32 or head_norm2_max.numel() != 1
                                        or head_norm2_max.device != x.device):
         raise ValueError("head_norm2_max must be one fp32 value on the device of x")
@@ -409,6 +468,8 @@ def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Option
         if t is None:
             return None
         t = t.reshape(-1, D)  # a view for (B,D), (B,1,D) and chunk() slices of a (B,k*D) projection
+        if t.dtype != _BF16:
+            t = t.to(_BF16)
         if t.stride(1) != 1:
             t = t.contiguous()
         if t.shape[0] not in (1, B):
@@ -420,6 +481,11 @@ def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Option
         return t
 
     scale_t, shift_t = prep(scale), prep(shift)
+    if any(t is not None and t.numel() != D for t in (ln_weight, ln_bias)):
+        raise ValueError("adaln_modulate: the LayerNorm affine has D = %d entries" % D)
+    ln_weight = None if ln_weight is None else ln_weight.to(_BF16).contiguous()
+    ln_bias = None if ln_bias is None else ln_bias.to(_BF16).contiguous()
+    _require_cuda(scale_t, shift_t, ln_weight, ln_bias)
     y = torch.empty((rows, D), dtype=_BF16, device=x.device) if want_bf16 else None
     q = torch.empty((rows, D), dtype=FP8, device=x.device) if want_fp8 else None
     qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
@@ -438,7 +504,9 @@ def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Option
 def gated_residual(x: torch.Tensor, y: torch.Tensor, gate: Optional[torch.Tensor],
                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x + gate * y (gate (B,D) / (B,1,D) or None); bf16, rounding bf16(x + bf16(gate*y))."""
-    _require_cuda(x, y)
+    _require_cuda(x, y, gate, out)
+    if x.dtype != _BF16 or y.dtype != _BF16 or x.shape != y.shape:
+        raise ValueError("gated_residual expects two bf16 tensors of one shape")
     shp = x.shape
     D = shp[-1]
     B = shp[0] if x.dim() == 3 else 1
@@ -448,6 +516,10 @@ def gated_residual(x: torch.Tensor, y: torch.Tensor, gate: Optional[torch.Tensor
     gate_sb = 0
     if gate is not None:
         gate = gate.reshape(-1, D)
+        if gate.shape[0] not in (1, B):
+            raise ValueError("gated_residual: the gate must have one row per batch entry")
+        if gate.dtype != _BF16:
+            gate = gate.to(_BF16)
         if gate.stride(1) != 1:
             gate = gate.contiguous()
         gate_sb = gate.stride(0) if gate.shape[0] > 1 else 0
