@@ -10,11 +10,16 @@ Two quantisation modes, chosen per weight:
     GEMM scales are 1.0 (what fp8_linear.py:35-48 computes);
   * scaled (default of ``enable_fp8_linear`` here): the Linear module gets a buffer ``weight_scale``
     (absmax/448, 0-dim fp32) and activations get a dynamic per-token scale.
-``F.linear(input, weight, bias)`` has no slot for a scale, so the weight Parameter carries a weak
-reference to its module (``_dsx_owner``) and the patched linear reads the buffer through it.  The buffer
-is module state: it follows ``.to()``, is written by ``state_dict()`` as ``<name>.weight_scale`` (the key
-the block runners look for) and is restored in place by ``load_state_dict``.
+``F.linear(input, weight, bias)`` has no slot for a scale.  The buffer is module state: it follows ``.to()``
+and ``copy.deepcopy``, is written by ``state_dict()`` as ``<name>.weight_scale`` (the key the block runners
+look for) and is restored in place by ``load_state_dict``.  It reaches the patched linear two ways:
+``fp8_inference`` also wraps ``nn.Linear.forward`` (the reference's LoRALinear calls it through ``super()``,
+models/basic/lora.py:137-141), which announces the module's buffer for the ``F.linear`` call it makes, so
+whatever else is chained onto ``F.linear`` still runs; and for code that calls ``F.linear(x, m.weight, m.bias)``
+itself the weight Parameter carries a weak reference to its module (``_dsx_owner``; ``enable_fp8_linear`` on an
+already converted module renews it, e.g. after a ``deepcopy``, which drops Parameter attributes).
 """
+import threading
 import weakref
 from contextlib import contextmanager
 
@@ -42,17 +47,44 @@ def _enable_fp8_linear(module: nn.Module, scaled: bool = True):
         if scale is not None:
             module.register_buffer(SCALE_BUFFER, scale)
             setattr(module.weight, OWNER_ATTR, weakref.ref(module))
+    elif isinstance(module, nn.Linear) and module.weight.data.dtype == ops.FP8 \
+            and module._buffers.get(SCALE_BUFFER) is not None:
+        setattr(module.weight, OWNER_ATTR, weakref.ref(module))  # converted earlier (and perhaps copied since)
     for submodule in module.children():
         _enable_fp8_linear(submodule, scaled)
 
 
+_announced = threading.local()  # (weight, scale) of the nn.Linear.forward call in progress on this thread
+
+
+def _linear_forward(self, input):
+    """nn.Linear.forward while fp8_inference is active: the same F.linear call, with the module's scale announced."""
+    scale = self._buffers.get(SCALE_BUFFER)
+    if scale is None:
+        return F.linear(input, self.weight, self.bias)
+    previous = getattr(_announced, "pair", None)
+    _announced.pair = (self.weight, scale)
+    try:
+        return F.linear(input, self.weight, self.bias)
+    finally:
+        _announced.pair = previous
+
+
 def weight_scale_of(weight: torch.Tensor):
     """The per-tensor scale that belongs to ``weight`` (None: a reference-style weight with unit scale)."""
-    owner = getattr(weight, OWNER_ATTR, None)
-    module = owner() if owner is not None else None
-    if module is None:
-        return None
-    scale = getattr(module, SCALE_BUFFER, None)
+    pair = getattr(_announced, "pair", None)
+    if pair is not None and pair[0] is weight:
+        scale = pair[1]
+    else:
+        owner = getattr(weight, OWNER_ATTR, None)
+        if owner is None:
+            return None
+        module = owner()
+        if module is None:
+            raise RuntimeError("the Linear module this scaled float8 weight was converted in is gone; its scale "
+                               "went with it (keep the module, or call enable_fp8_linear on the one that holds "
+                               "the weight now)")
+        scale = module._buffers.get(SCALE_BUFFER)
     if scale is not None and scale.device != weight.device:
         raise RuntimeError("weight_scale of a Linear is on %s, its weight on %s" % (scale.device, weight.device))
     return scale
@@ -80,9 +112,11 @@ def fp8_inference(enabled=True):
     if not enabled:
         yield
         return
-    origin_linear = F.linear
+    origin_linear, origin_forward = F.linear, nn.Linear.forward
     F.linear = fp8_linear
+    nn.Linear.forward = _linear_forward
     try:
         yield
     finally:
         F.linear = origin_linear
+        nn.Linear.forward = origin_forward

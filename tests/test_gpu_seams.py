@@ -120,3 +120,39 @@ def test_weight_scale_travels_with_the_module_state(dev):
     del sd["net.0.weight_scale"]
     with pytest.raises(ValueError, match="net.0"):
         ingest_state_dict(sd, dev, scaled=True)
+
+
+def test_weight_scale_survives_deepcopy_and_a_dead_owner_is_an_error(dev):
+    """copy.deepcopy drops Python attributes of a Parameter, the buffer it keeps: under fp8_inference the copy
+    computes what the original does (through nn.Linear.forward, which announces the module's scale).  A direct
+    F.linear call with a scaled weight whose module is gone raises instead of running at unit scale, and
+    enable_fp8_linear on the copy renews the link for such callers."""
+    import copy
+    import gc
+
+    from diffsynth_engine_amd import enable_fp8_linear, fp8_inference
+
+    torch.manual_seed(11)
+    m = _Mlp().to(torch.bfloat16).to(dev)
+    enable_fp8_linear(m)
+    x = torch.randn(24, 256, generator=torch.Generator().manual_seed(12)).bfloat16().to(dev)
+    forward_before, linear_before = nn.Linear.forward, F.linear
+    with fp8_inference():
+        assert F.linear is not linear_before
+        want = m(x)
+        direct = F.linear(x, m.net[0].weight, m.net[0].bias)
+        assert torch.equal(direct, m.net[0](x))
+    c = copy.deepcopy(m)
+    assert not hasattr(c.net[0].weight, "_dsx_owner") and c.net[0].weight_scale.item() == m.net[0].weight_scale.item()
+    with fp8_inference():
+        assert torch.equal(c(x), want)
+    assert nn.Linear.forward is forward_before and F.linear is linear_before
+    enable_fp8_linear(c)  # already converted: only the link is renewed
+    with fp8_inference():
+        assert torch.equal(F.linear(x, c.net[0].weight, c.net[0].bias), direct)
+    w, b = m.net[0].weight, m.net[0].bias
+    del m
+    gc.collect()
+    with fp8_inference():
+        with pytest.raises(RuntimeError, match="scale"):
+            F.linear(x, w, b)
