@@ -21,7 +21,7 @@ DSX_EARCH = -3
 DSX_ELAUNCH = -4
 DSX_ENULL = -5
 DSX_EWORKSPACE = -6
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class AttnParams(ctypes.Structure):
@@ -112,6 +112,8 @@ SIGNATURES = {
                                    c_int64, c_int64, c_int64, c_void_p]),
     "dsx_gelu_tanh": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64,
                               c_void_p]),
+    "dsx_gelu_erf": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64,
+                             c_void_p]),
     "dsx_flow_match_euler_step": (c_int, [c_void_p, c_void_p, c_float, c_void_p, c_int64, c_int, c_void_p]),
     "dsx_mfma_ceiling_probe": (c_int, [c_int, c_void_p, c_int64, ctypes.c_int32, c_void_p, ctypes.POINTER(c_int64),
                                        c_void_p]),

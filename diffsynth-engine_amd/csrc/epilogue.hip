@@ -302,10 +302,13 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const uint16_t* __res
   }
 }
 
-// tanh-GELU of x, optionally preceded in the OUTPUT row by an unmodified prefix:
+// erf-GELU as torch evaluates nn.GELU() in fp32: x * 0.5 * (1 + erf(x / sqrt(2))).
+__device__ __forceinline__ float gelu_erf_f32(float x) { return x * 0.5f * (1.0f + erff(x * 0.70710678118654752f)); }
+
+// GELU (tanh form, or the erf form with ERF) of x, optionally preceded in the OUTPUT row by an unmodified prefix:
 // out row = [ prefix (Dp) | gelu(x) (D) ].  The prefix form is the single-stream block's
 // cat([attention, gelu(mlp)]) built directly in the operand format of proj_out.
-template <int NCH>
+template <int NCH, bool ERF>
 __global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restrict__ prefix, int64_t ldp,
                                                         int Dp, const uint16_t* __restrict__ x, int64_t ldx,
                                                         uint16_t* __restrict__ y, int64_t ldy,
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restri
     unpack8(raw[i], val[i]);
     if (c >= npre) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(gelu_tanh_f32(val[i][j]));
+      for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(ERF ? gelu_erf_f32(val[i][j]) : gelu_tanh_f32(val[i][j]));
     }
     if (c >= nchunk) {
 #pragma unroll
@@ -429,22 +432,23 @@ extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale,
 
 static int launch_gelu(const void* prefix, int64_t ldp, int64_t Dp, const void* x, int64_t ldx, void* y,
                        int64_t ldy, void* q, int64_t ldq, float* q_scale, int64_t rows, int64_t D,
-                       hipStream_t st) {
+                       hipStream_t st, bool erf = false) {
   using namespace dsx;
   const int64_t Dt = Dp + D;
   dim3 grid((unsigned)rows), block(256);
-#define DSX_LAUNCH_GELU(NCH)                                                                        \
-  gelu_tanh_kernel<NCH><<<grid, block, 0, st>>>((const uint16_t*)prefix, ldp, (int)Dp, (const uint16_t*)x, \
-                                                ldx, (uint16_t*)y, ldy, (uint8_t*)q, ldq, q_scale, (int)D)
-  if (Dt <= 2048 * 2) DSX_LAUNCH_GELU(2);
-  else if (Dt <= 2048 * 6) DSX_LAUNCH_GELU(6);
-  else DSX_LAUNCH_GELU(8);
+#define DSX_LAUNCH_GELU(NCH, ERF)                                                                             \
+  gelu_tanh_kernel<NCH, ERF><<<grid, block, 0, st>>>((const uint16_t*)prefix, ldp, (int)Dp, (const uint16_t*)x, \
+                                                     ldx, (uint16_t*)y, ldy, (uint8_t*)q, ldq, q_scale, (int)D)
+  if (erf) DSX_LAUNCH_GELU(8, true);  // (the erf form serves a 257-row embedder: one instantiation is enough)
+  else if (Dt <= 2048 * 2) DSX_LAUNCH_GELU(2, false);
+  else if (Dt <= 2048 * 6) DSX_LAUNCH_GELU(6, false);
+  else DSX_LAUNCH_GELU(8, false);
 #undef DSX_LAUNCH_GELU
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
-extern "C" int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
-                             float* q_scale, int64_t rows, int64_t D, void* stream) {
+static int gelu_plain(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq, float* q_scale,
+                      int64_t rows, int64_t D, void* stream, bool erf) {
   using namespace dsx;
   if (rows == 0) return DSX_OK;  // an empty batch has no buffers to point at
   if (!x || (!y && !q) || (q && !q_scale)) return DSX_ENULL;
@@ -453,8 +457,17 @@ extern "C" int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, v
   if ((ldx & 7) || (y && (ldy & 7)) || (q && (ldq & 7)) || misaligned16(x) || misaligned16(y) ||
       ((uintptr_t)q & 7))
     return DSX_EALIGN;
-  if (rows == 0) return DSX_OK;
-  return launch_gelu(x, 0, 0, x, ldx, y, ldy, q, ldq, q_scale, rows, D, (hipStream_t)stream);
+  return launch_gelu(x, 0, 0, x, ldx, y, ldy, q, ldq, q_scale, rows, D, (hipStream_t)stream, erf);
+}
+
+extern "C" int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
+                             float* q_scale, int64_t rows, int64_t D, void* stream) {
+  return gelu_plain(x, ldx, y, ldy, q, ldq, q_scale, rows, D, stream, false);
+}
+
+extern "C" int dsx_gelu_erf(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
+                            float* q_scale, int64_t rows, int64_t D, void* stream) {
+  return gelu_plain(x, ldx, y, ldy, q, ldq, q_scale, rows, D, stream, true);
 }
 
 extern "C" int dsx_concat_gelu_tanh(const void* prefix, int64_t ldp, int64_t Dp, const void* x, int64_t ldx,

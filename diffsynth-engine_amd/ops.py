@@ -534,9 +534,11 @@ def gated_residual(x: torch.Tensor, y: torch.Tensor, gate: Optional[torch.Tensor
     return out.view(shp)
 
 
-def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, out: Optional[torch.Tensor] = None):
-    """tanh-GELU over the last dim of a bf16 tensor (a column slice of a wider buffer is fine)."""
-    _require_cuda(x)
+def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, out: Optional[torch.Tensor] = None,
+              erf: bool = False):
+    """tanh-GELU (``erf``: the exact erf form of nn.GELU()) over the last dim of a bf16 tensor (a column slice of
+    a wider buffer is fine)."""
+    _require_cuda(x, out)
     if x.dtype != _BF16:
         raise ValueError("gelu_tanh expects bf16")
     shp = x.shape
@@ -551,8 +553,9 @@ def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, o
             y = torch.empty((rows, D), dtype=_BF16, device=x.device)
     q = torch.empty((rows, D), dtype=FP8, device=x.device) if want_fp8 else None
     qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
-    rc = _lib.load().dsx_gelu_tanh(_ptr(x2), ldx, _ptr(y), ldy, _ptr(q), D, _ptr(qs), rows, D, _stream())
-    _lib.check(rc, "dsx_gelu_tanh")
+    fn = _lib.load().dsx_gelu_erf if erf else _lib.load().dsx_gelu_tanh
+    _lib.check(fn(_ptr(x2), ldx, _ptr(y), ldy, _ptr(q), D, _ptr(qs), rows, D, _stream()),
+               "dsx_gelu_erf" if erf else "dsx_gelu_tanh")
     res = []
     if want_bf16:
         res.append(out if out is not None else y.view(shp))

@@ -1,4 +1,5 @@
-"""Fused MI355X runner of the Wan2.1 DiT denoising step (text-to-video variant).
+"""Fused MI355X runner of the Wan2.1 DiT denoising step (text-to-video, and image-to-video when the checkpoint
+holds the ``has_image_input`` entries).
 
 Same inputs/outputs and state-dict names as ``WanDiT.forward``
 (diffsynth_engine/models/wan/wan_dit.py:319-351).  ``DiTBlock.forward`` (:185-193) is issued as:
@@ -8,6 +9,11 @@ Same inputs/outputs and state-dict names as ``WanDiT.forward``
   residual in its epilogue -> LayerNorm(affine) (+ e4m3) -> cross-attention against the text keys/values
   (Lq != Lk) -> o GEMM with plain residual -> AdaLN-modulate -> FFN GEMM -> GELU (+ e4m3) -> FFN GEMM with
   gated residual.
+
+Image-to-video (conf/models/wan/dit/14b-i2v.json; wan_dit.py:136-152,195-211,329-333): the encoded image rides
+along as extra latent channels, the CLIP feature goes through the ``img_emb`` MLP and its 257 rows are put in
+front of the text context, and every cross-attention adds a second attention of the same queries over those rows
+(own k/v projections and k norm) before the o projection.
 
 The reference wires FP8 for Flux only (models/flux/flux_dit.py:404; pipelines/base.py:164-165 raises for the
 rest); here every Linear of the Wan DiT runs through the same scaled e4m3 GEMM as Flux.
@@ -19,6 +25,9 @@ import torch
 
 from . import ops
 from .flux_dit import _Linear, ingest_state_dict
+
+
+IMAGE_ROWS = 257  # CLIP tokens in front of the text context (the split is hard-coded, wan_dit.py:138-139)
 
 
 class WanDiTRunner:
@@ -37,6 +46,7 @@ class WanDiTRunner:
         # key order does not matter: biases are attached once every weight is known; what is not a Linear
         # (modulation vectors, norm weights and the affine bias of norm3) lands in `vec` under its full key
         self.lin, self.vec = ingest_state_dict(state_dict, self.device, scaled, as_linear=conv_as_linear)
+        self.has_image_input = "img_emb.proj.1" in self.lin
 
     # ------------------------------------------------------------------ helpers
     def _linear_bf16(self, x, name):
@@ -108,11 +118,22 @@ class WanDiTRunner:
         hq, hs = self._modulate_q(x2.view(B, S, d), None, None, V[p + "norm3.weight"], V[p + "norm3.bias"])
         q = ops.rmsnorm_rows(L[p + "cross_attn.q"](hq.view(B * S, d), hs).view(B, S, d),
                              V[p + "cross_attn.norm_q.weight"], eps)
+        img = None
+        if self.has_image_input:  # [257 embedded CLIP rows | text rows] (CrossAttention.forward, wan_dit.py:136-152)
+            img, context = context[:, :IMAGE_ROWS], context[:, IMAGE_ROWS:]
         Sc = context.shape[1]
         cq, cs = self._q(context.reshape(B * Sc, d))
         k = ops.rmsnorm_rows(L[p + "cross_attn.k"](cq, cs).view(B, Sc, d), V[p + "cross_attn.norm_k.weight"], eps)
         v = L[p + "cross_attn.v"](cq, cs).view(B, Sc, d)
-        aq, asc = self._q(self._attention(q, k, v))
+        a = self._attention(q, k, v)
+        if img is not None:  # the same queries over the image rows; the two outputs are added in bf16
+            Si = img.shape[1]
+            iq, isc = self._q(img.reshape(B * Si, d))
+            k = ops.rmsnorm_rows(L[p + "cross_attn.k_img"](iq, isc).view(B, Si, d),
+                                 V[p + "cross_attn.norm_k_img.weight"], eps)
+            v = L[p + "cross_attn.v_img"](iq, isc).view(B, Si, d)
+            a = ops.gated_residual(a, self._attention(q, k, v), None)
+        aq, asc = self._q(a)
         x2 = L[p + "cross_attn.o"](aq, asc, resid=x2, gate=None, rows_per_batch=S)
         # feed-forward
         hq, hs = self._modulate_q(x2.view(B, S, d), m[4], m[3])
@@ -125,8 +146,18 @@ class WanDiTRunner:
         return x2.view(B, S, d)
 
     # ------------------------------------------------------------------ step
+    def _img_emb(self, clip_feature):
+        """MLP.forward (wan_dit.py:195-211): LayerNorm (affine, eps 1e-5) -> Linear -> erf-GELU -> Linear -> LayerNorm."""
+        V = self.vec
+        h = ops.adaln_modulate(clip_feature.to(torch.bfloat16), None, None, 1e-5, ln_weight=V["img_emb.proj.0.weight"],
+                               ln_bias=V["img_emb.proj.0.bias"])
+        h = self._linear_bf16(ops.gelu_tanh(self._linear_bf16(h, "img_emb.proj.1"), erf=True), "img_emb.proj.3")
+        return ops.adaln_modulate(h, None, None, 1e-5, ln_weight=V["img_emb.proj.4.weight"],
+                                  ln_bias=V["img_emb.proj.4.bias"])
+
     @torch.no_grad()
-    def forward(self, x, context, timestep):
+    def forward(self, x, context, timestep, clip_feature=None, y=None):
+        """``clip_feature`` (B,257,clip_dim) and ``y`` (B,c_y,f,h,w): the image-to-video inputs (both or neither)."""
         cfg = self.cfg
         d = cfg["dim"]
         pf, ph, pw = cfg["patch_size"]
@@ -139,6 +170,13 @@ class WanDiTRunner:
         t_mod = self._linear_bf16(torch.nn.functional.silu(t), "time_projection.1").unflatten(1, (6, d))
         ctx = ops.gelu_tanh(self._linear_bf16(context.to(bf), "text_embedding.0"))
         ctx = self._linear_bf16(ctx, "text_embedding.2")
+        if self.has_image_input != (clip_feature is not None and y is not None):
+            raise ValueError("clip_feature and y go with an image-to-video checkpoint, and only with one")
+        if self.has_image_input:
+            if clip_feature.shape[1] != IMAGE_ROWS:
+                raise ValueError("clip_feature must have %d rows, got %d" % (IMAGE_ROWS, clip_feature.shape[1]))
+            x = torch.cat([x, y.to(x.dtype)], dim=1)                         # (b, c_x + c_y, f, h, w)  (:331)
+            ctx = torch.cat([self._img_emb(clip_feature), ctx], dim=1)  # image rows first           (:333)
         B, C, Fr, Hh, Ww = x.shape
         f, h, w = Fr // pf, Hh // ph, Ww // pw
         patches = x.to(bf).view(B, C, f, pf, h, ph, w, pw).permute(0, 2, 4, 6, 1, 3, 5, 7)

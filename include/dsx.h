@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define DSX_ABI_VERSION 5
+#define DSX_ABI_VERSION 6
 
 enum {
   DSX_OK = 0,
@@ -316,6 +316,13 @@ int dsx_gated_residual(const void* x, int64_t ldx, const void* y, int64_t ldy, c
  */
 int dsx_gelu_tanh(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
                   float* q_scale, int64_t rows, int64_t D, void* stream);
+
+/*
+ * erf-GELU, same arguments: y = bf16(x * 0.5 * (1 + erf(x / sqrt(2)))) in fp32.  Replaces the nn.GELU() of the
+ * image-to-video CLIP embedder (models/wan/wan_dit.py:195-211, MLP.proj[2]).
+ */
+int dsx_gelu_erf(const void* x, int64_t ldx, void* y, int64_t ldy, void* q, int64_t ldq,
+                 float* q_scale, int64_t rows, int64_t D, void* stream);
 
 /*
  * Concatenating tanh-GELU: output row = [ prefix (Dp, copied) | gelu_tanh(x) (D) ], emitted as bf16

@@ -1,9 +1,10 @@
 """Wan2.1 DiT block and model forward — oracle (test infrastructure, see oracle/__init__.py).
 
-Restates diffsynth_engine/models/wan/wan_dit.py:18-351 (text-to-video variant, has_image_input=False) as
-functions over a flat parameter dict whose keys are the reference's state-dict names.  The reference has
-no WanDiT test; wiring is pinned by vectors its own WanDiT class wrote at reduced size
-(tests/test_oracle_leaf_goldens.py) and by structural invariants (tests/test_oracle_wan.py).  ``linear_mode`` as in oracle/flux.py.
+Restates diffsynth_engine/models/wan/wan_dit.py:18-351 (text-to-video, and image-to-video where the parameter
+dict holds the has_image_input=True entries) as functions over a flat parameter dict whose keys are the
+reference's state-dict names.  The reference has no WanDiT test; wiring is pinned by vectors its own WanDiT
+class wrote at reduced size in both forms (tests/test_oracle_leaf_goldens.py) and by structural invariants
+(tests/test_oracle_wan.py).  ``linear_mode`` as in oracle/flux.py.
 """
 import math
 
@@ -20,8 +21,13 @@ def config_14b():
                 patch_size=(1, 2, 2), num_heads=40, num_layers=40)
 
 
-def init_params(cfg, dtype=torch.bfloat16, device="cpu", seed=0, std=0.02, bias_std=0.0):
-    """Random WanDiT parameters (shapes from WanDiT.__init__, wan_dit.py:248-299)."""
+IMAGE_ROWS = 257  # CLIP tokens in front of the text context (the split is hard-coded, wan_dit.py:138-139)
+
+
+def init_params(cfg, dtype=torch.bfloat16, device="cpu", seed=0, std=0.02, bias_std=0.0, clip_dim=None):
+    """Random WanDiT parameters (shapes from WanDiT.__init__, wan_dit.py:248-299); with ``clip_dim`` the
+    image-to-video form (cross_attn.k_img / v_img / norm_k_img per block and the img_emb MLP, 1280 wide in the
+    reference)."""
     g = torch.Generator(device="cpu").manual_seed(seed)
     d, f = cfg["dim"], cfg["ffn_dim"]
     t = {}
@@ -48,11 +54,21 @@ def init_params(cfg, dtype=torch.bfloat16, device="cpu", seed=0, std=0.02, bias_
             t[p + f"{a}.norm_k.weight"] = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype).to(device)
         t[p + "norm3.weight"] = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype).to(device)
         t[p + "norm3.bias"] = (0.1 * torch.randn(d, generator=g)).to(dtype).to(device)
+        if clip_dim:
+            lin(p + "cross_attn.k_img", d, d)
+            lin(p + "cross_attn.v_img", d, d)
+            t[p + "cross_attn.norm_k_img.weight"] = (1 + 0.1 * torch.randn(d, generator=g)).to(dtype).to(device)
         lin(p + "ffn.0", d, f)
         lin(p + "ffn.2", f, d)
         t[p + "modulation"] = (torch.randn(1, 6, d, generator=g) / d ** 0.5).to(dtype).to(device)
     lin("head.head", d, cfg["out_dim"] * pf * ph * pw)
     t["head.modulation"] = (torch.randn(1, 2, d, generator=g) / d ** 0.5).to(dtype).to(device)
+    if clip_dim:
+        for i, n in ((0, clip_dim), (4, d)):
+            t[f"img_emb.proj.{i}.weight"] = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype).to(device)
+            t[f"img_emb.proj.{i}.bias"] = (0.1 * torch.randn(n, generator=g)).to(dtype).to(device)
+        lin("img_emb.proj.1", clip_dim, clip_dim)
+        lin("img_emb.proj.3", clip_dim, d)
     return t
 
 
@@ -107,9 +123,16 @@ def dit_block(P, i, x, context, t_mod, freqs, cfg, attn=O.sdpa):
     x = x + gate_msa * P.linear(a, p + "self_attn.o")
     h = O.layer_norm_modulate(x, None, None, eps, P[p + "norm3.weight"], P[p + "norm3.bias"])
     q = wan_rms_norm(P.linear(h, p + "cross_attn.q"), P[p + "cross_attn.norm_q.weight"], eps)
-    k = wan_rms_norm(P.linear(context, p + "cross_attn.k"), P[p + "cross_attn.norm_k.weight"], eps)
-    v = P.linear(context, p + "cross_attn.v")
-    x = x + P.linear(attention(q, k, v, H, attn), p + "cross_attn.o")
+    # CrossAttention.forward (wan_dit.py:136-152): with image input the first 257 context rows are the embedded
+    # CLIP tokens; they get their own k/v projections and k norm, and the two attention outputs are added
+    img, ctx = (context[:, :IMAGE_ROWS], context[:, IMAGE_ROWS:]) if p + "cross_attn.k_img.weight" in P.t else (None, context)
+    k = wan_rms_norm(P.linear(ctx, p + "cross_attn.k"), P[p + "cross_attn.norm_k.weight"], eps)
+    v = P.linear(ctx, p + "cross_attn.v")
+    a = attention(q, k, v, H, attn)
+    if img is not None:
+        k_img = wan_rms_norm(P.linear(img, p + "cross_attn.k_img"), P[p + "cross_attn.norm_k_img.weight"], eps)
+        a = a + attention(q, k_img, P.linear(img, p + "cross_attn.v_img"), H, attn)
+    x = x + P.linear(a, p + "cross_attn.o")
     h = O.layer_norm_modulate(x, scale_mlp, shift_mlp, eps)
     return x + gate_mlp * P.linear(O.gelu_tanh(P.linear(h, p + "ffn.0")), p + "ffn.2")
 
@@ -122,14 +145,26 @@ def sinusoidal_embedding_1d(dim, position):
     return torch.cat([torch.cos(ang), torch.sin(ang)], dim=1).to(position.dtype)
 
 
-def wan_dit_forward(P, x, context, timestep, cfg, attn=O.sdpa):
-    """WanDiT.forward (wan_dit.py:319-351), text-to-video."""
+def img_emb(P, clip_feature):
+    """MLP.forward (wan_dit.py:195-211): LayerNorm (affine, eps 1e-5) -> Linear -> erf-GELU -> Linear -> LayerNorm."""
+    n = clip_feature.shape[-1]
+    h = F.layer_norm(clip_feature, (n,), P["img_emb.proj.0.weight"], P["img_emb.proj.0.bias"], 1e-5)
+    h = P.linear(F.gelu(P.linear(h, "img_emb.proj.1")), "img_emb.proj.3")
+    return F.layer_norm(h, (h.shape[-1],), P["img_emb.proj.4.weight"], P["img_emb.proj.4.bias"], 1e-5)
+
+
+def wan_dit_forward(P, x, context, timestep, cfg, attn=O.sdpa, clip_feature=None, y=None):
+    """WanDiT.forward (wan_dit.py:319-351); ``clip_feature`` (B,257,clip_dim) and ``y`` (B,c_y,f,h,w) for the
+    image-to-video form."""
     d = cfg["dim"]
     pf, ph, pw = cfg["patch_size"]
     t = P.linear(F.silu(P.linear(sinusoidal_embedding_1d(cfg["freq_dim"], timestep), "time_embedding.0")),
                  "time_embedding.2")
     t_mod = P.linear(F.silu(t), "time_projection.1").unflatten(1, (6, d))
     context = P.linear(F.gelu(P.linear(context, "text_embedding.0"), approximate="tanh"), "text_embedding.2")
+    if clip_feature is not None:
+        x = torch.cat([x, y], dim=1)                                   # (b, c_x + c_y, f, h, w)  (:331)
+        context = torch.cat([img_emb(P, clip_feature), context], dim=1)  # image rows first           (:333)
     # Conv3d with kernel == stride is a Linear over each (c, pf, ph, pw) patch
     B, C, Fr, Hh, Ww = x.shape
     f, h, w = Fr // pf, Hh // ph, Ww // pw

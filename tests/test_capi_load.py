@@ -32,7 +32,7 @@ def test_abi_version_and_strerror():
     from diffsynth_engine_amd import _lib
 
     lib = _lib.load()
-    assert lib.dsx_abi_version() == 5
+    assert lib.dsx_abi_version() == 6
     assert _lib.strerror(0) == "ok"
     for code in (-1, -2, -3, -4, -5, -6):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)

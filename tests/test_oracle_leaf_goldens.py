@@ -151,6 +151,54 @@ def test_wan_model_forward_against_reference_vectors():
     _close(got, W["model.out"], 5e-5)
 
 
+# ---- WanDiT, image-to-video form (has_image_input=True; tests/golden/make_wan_i2v_fixtures.py)
+WI = load_file(os.path.join(os.path.dirname(__file__), "golden", "wan_i2v.safetensors"))
+WICFG = dict(WCFG, in_dim=8)
+
+
+def _wiparams(drop=()):
+    from oracle import wan as OW
+    return OW, OW.Params({k[6:]: v.clone() for k, v in WI.items() if k.startswith("param.") and
+                          not any(d in k for d in drop)})
+
+
+def test_wan_i2v_img_emb_against_reference_vectors():
+    OW, P = _wiparams()
+    _close(OW.img_emb(P, WI["model.clip_feature"]), WI["img_emb.out"], 2e-5)
+    # tanh-GELU in place of the erf form is a different function at this bar
+    import torch.nn.functional as F
+    h = F.layer_norm(WI["model.clip_feature"], (24,), P["img_emb.proj.0.weight"], P["img_emb.proj.0.bias"], 1e-5)
+    h = P.linear(F.gelu(P.linear(h, "img_emb.proj.1"), approximate="tanh"), "img_emb.proj.3")
+    wrong = F.layer_norm(h, (40,), P["img_emb.proj.4.weight"], P["img_emb.proj.4.bias"], 1e-5)
+    assert (wrong - WI["img_emb.out"]).abs().max() > 1e-3
+
+
+def test_wan_i2v_block_against_reference_vectors():
+    OW, P = _wiparams()
+    freqs = torch.view_as_complex(WI["block.freqs_real"])
+    got = OW.dit_block(P, 1, WI["block.x"], WI["block.context"], WI["block.t_mod"], freqs, WICFG)
+    _close(got, WI["block.out"], 2e-5)
+    # negative controls: without the image branch (all 262 rows as text), and with the image rows taken from the
+    # END of the context instead of its first 257 rows, the block is a different function
+    _, Pt = _wiparams(drop=("k_img", "v_img"))
+    assert (OW.dit_block(Pt, 1, WI["block.x"], WI["block.context"], WI["block.t_mod"], freqs, WICFG)
+            - WI["block.out"]).abs().max() > 1e-2
+    swapped = torch.cat([WI["block.context"][:, 257:], WI["block.context"][:, :257]], dim=1)
+    assert (OW.dit_block(P, 1, WI["block.x"], swapped, WI["block.t_mod"], freqs, WICFG)
+            - WI["block.out"]).abs().max() > 1e-2
+
+
+def test_wan_i2v_model_forward_against_reference_vectors():
+    OW, P = _wiparams()
+    got = OW.wan_dit_forward(P, WI["model.x"], WI["model.context"], WI["model.timestep"], WICFG,
+                             clip_feature=WI["model.clip_feature"], y=WI["model.y"])
+    _close(got, WI["model.out"], 5e-5)
+    # channel order of the concat: [x | y], not [y | x]
+    wrong = OW.wan_dit_forward(P, WI["model.y"], WI["model.context"], WI["model.timestep"], WICFG,
+                               clip_feature=WI["model.clip_feature"], y=WI["model.x"])
+    assert (wrong - WI["model.out"]).abs().max() > 1e-2
+
+
 # ---- the reference's fp8 patch of F.linear (diffsynth_engine/utils/fp8_linear.py) on one nn.Linear
 def test_reference_fp8_linear_vectors():
     from oracle import fp8
