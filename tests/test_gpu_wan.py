@@ -99,6 +99,26 @@ def test_two_layers_at_the_14b_width(dev):
     assert c >= 0.99 and c >= min(0.999, floor - 1e-3), (c, floor)
 
 
+def test_block_at_the_1_3b_width(dev):
+    """conf/models/wan/dit/1.3b-t2v.json: dim 1536 = 12 heads x 128, FFN 8960.  One block teacher-forced at
+    3 x 30 x 52 = 4680 video tokens + 512 text tokens against the oracle evaluated by torch on the device: the
+    64-lanes-per-row form of the full-width RMSNorm and GEMMs with K = 1536 and 8960 in a model."""
+    from bench import wan_state_dict_stream
+    from diffsynth_engine_amd.wan_dit import WanDiTRunner
+
+    cfg = dict(ow.config_14b(), dim=1536, ffn_dim=8960, num_heads=12, num_layers=1)
+    sd = dict(wan_state_dict_stream(cfg, dev, seed=2))
+    g = torch.Generator(device=dev).manual_seed(9)
+    f, h, w = 3, 30, 52
+    x = torch.randn(1, f * h * w, 1536, generator=g, device=dev).bfloat16()
+    ctx = torch.randn(1, 512, 1536, generator=g, device=dev).bfloat16()
+    t_mod = (torch.randn(1, 6, 1536, generator=g, device=dev) * 0.3).bfloat16()
+    R = WanDiTRunner(sd, cfg, scaled=True, device=dev)
+    got = R.block(0, x, ctx, t_mod, R.rope_table(f, h, w))
+    want = ow.dit_block(ow.Params(sd, "fp8_scaled"), 0, x, ctx, t_mod, ow.freqs_cis_3d(128, f, h, w).to(dev), cfg)
+    assert _cos(got, want) >= 0.9995, _cos(got, want)
+
+
 @pytest.mark.parametrize("S,D", [(24, 256), (1100, 1536), (700, 3072), (2049, 5120), (33, 8192)])
 def test_rmsnorm_rows_leaves_the_largest_squared_head_norm(dev, S, D):
     """head_norm2_max: every launch shape of the row kernel (64, 128 and 256 lanes per row) raises the float to
