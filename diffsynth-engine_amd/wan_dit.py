@@ -24,7 +24,7 @@ from typing import Dict
 import torch
 
 from . import ops
-from .flux_dit import _Linear, ingest_state_dict
+from .flux_dit import _Linear, _gemm_pair, ingest_state_dict
 
 
 IMAGE_ROWS = 257  # CLIP tokens in front of the text context (the split is hard-coded, wan_dit.py:138-139)
@@ -92,8 +92,22 @@ class WanDiTRunner:
         return out.view(B * Sq, HD)
 
     # ------------------------------------------------------------------ block
-    def block(self, i, x, context, t_mod, rope):
-        """DiTBlock.forward; x (B,S,d), context (B,Sc,d) already embedded, t_mod (B,6,d)."""
+    def quantise_context(self, context):
+        """The cross-attention operand of every block: the embedded context as e4m3 rows with their scales, text
+        rows and (image-to-video) the 257 CLIP rows in front of them separately (CrossAttention.forward,
+        wan_dit.py:136-152).  The same for every block of a step, so the step does it once."""
+        B, _, d = context.shape
+        img = None
+        if self.has_image_input:
+            img, context = context[:, :IMAGE_ROWS], context[:, IMAGE_ROWS:]
+        parts = []
+        for t in (context, img):
+            parts.append(None if t is None else self._q(t.reshape(B * t.shape[1], d)) + (t.shape[1],))
+        return parts
+
+    def block(self, i, x, context, t_mod, rope, context_q=None):
+        """DiTBlock.forward; x (B,S,d), context (B,Sc,d) already embedded, t_mod (B,6,d); ``context_q``: what
+        quantise_context(context) returned, when the caller has it already."""
         p = f"blocks.{i}."
         L, V, eps = self.lin, self.vec, self.cfg["eps"]
         B, S, d = x.shape
@@ -118,21 +132,17 @@ class WanDiTRunner:
         hq, hs = self._modulate_q(x2.view(B, S, d), None, None, V[p + "norm3.weight"], V[p + "norm3.bias"])
         q = ops.rmsnorm_rows(L[p + "cross_attn.q"](hq.view(B * S, d), hs).view(B, S, d),
                              V[p + "cross_attn.norm_q.weight"], eps)
-        img = None
-        if self.has_image_input:  # [257 embedded CLIP rows | text rows] (CrossAttention.forward, wan_dit.py:136-152)
-            img, context = context[:, :IMAGE_ROWS], context[:, IMAGE_ROWS:]
-        Sc = context.shape[1]
-        cq, cs = self._q(context.reshape(B * Sc, d))
-        k = ops.rmsnorm_rows(L[p + "cross_attn.k"](cq, cs).view(B, Sc, d), V[p + "cross_attn.norm_k.weight"], eps)
-        v = L[p + "cross_attn.v"](cq, cs).view(B, Sc, d)
-        a = self._attention(q, k, v)
+        # k and v projections of the context share their operand: one launch, side by side
+        (cq, cs, Sc), img = context_q if context_q is not None else self.quantise_context(context)
+        k, v = _gemm_pair(L[p + "cross_attn.k"], dict(a_q=cq, a_s=cs), L[p + "cross_attn.v"], dict(a_q=cq, a_s=cs))
+        k = ops.rmsnorm_rows(k.view(B, Sc, d), V[p + "cross_attn.norm_k.weight"], eps)
+        a = self._attention(q, k, v.view(B, Sc, d))
         if img is not None:  # the same queries over the image rows; the two outputs are added in bf16
-            Si = img.shape[1]
-            iq, isc = self._q(img.reshape(B * Si, d))
-            k = ops.rmsnorm_rows(L[p + "cross_attn.k_img"](iq, isc).view(B, Si, d),
-                                 V[p + "cross_attn.norm_k_img.weight"], eps)
-            v = L[p + "cross_attn.v_img"](iq, isc).view(B, Si, d)
-            a = ops.gated_residual(a, self._attention(q, k, v), None)
+            iq, isc, Si = img
+            k, v = _gemm_pair(L[p + "cross_attn.k_img"], dict(a_q=iq, a_s=isc),
+                              L[p + "cross_attn.v_img"], dict(a_q=iq, a_s=isc))
+            k = ops.rmsnorm_rows(k.view(B, Si, d), V[p + "cross_attn.norm_k_img.weight"], eps)
+            a = ops.gated_residual(a, self._attention(q, k, v.view(B, Si, d)), None)
         aq, asc = self._q(a)
         x2 = L[p + "cross_attn.o"](aq, asc, resid=x2, gate=None, rows_per_batch=S)
         # feed-forward
@@ -182,8 +192,9 @@ class WanDiTRunner:
         patches = x.to(bf).view(B, C, f, pf, h, ph, w, pw).permute(0, 2, 4, 6, 1, 3, 5, 7)
         hs = self._linear_bf16(patches.reshape(B, f * h * w, C * pf * ph * pw), "patch_embedding")
         rope = self.rope_table(f, h, w)
+        ctx_q = self.quantise_context(ctx)
         for i in range(cfg["num_layers"]):
-            hs = self.block(i, hs, ctx, t_mod, rope)
+            hs = self.block(i, hs, ctx, t_mod, rope, ctx_q)
         shift, scale = (self.vec["head.modulation"] + t).chunk(2, dim=1)  # Head.forward (wan_dit.py:234-237)
         hq, hsc = self._modulate_q(hs, scale.reshape(B, d), shift.reshape(B, d))
         out = self.lin["head.head"](hq.view(-1, d), hsc)
