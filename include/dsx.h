@@ -249,7 +249,8 @@ int64_t dsx_attn_static_scratch_bytes(void);
 /*
  * Standalone RMSNorm + RoPE of q and k (same arithmetic and rounding points as the fused
  * option of dsx_attn_fwd), written to a strided (B,H,S,128) bf16 view; `out` may be `x` itself
- * (in place).  One tensor per call.
+ * (in place).  One tensor per call.  Row s of every head takes table row rope_pos0 + s (+ rope_sb floats per batch
+ * entry): the table must hold rope_pos0 + seq rows of 128 floats per entry; the call cannot check that.
  * Replaces RMSNorm.forward (transformer_helper.py:73-78) followed by apply_rope (flux_dit.py:154-159).
  */
 int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss, const void* norm_w,
@@ -262,8 +263,9 @@ int dsx_rmsnorm_rope(const void* x, int64_t x_sb, int64_t x_sh, int64_t x_ss, co
  * projection in ONE pass: token row at x + b*x_sb + s*x_ss, head h of that token at + h*128,
  * heads [0, heads_q) normalised with q_norm_w, heads [heads_q, heads_q + heads_k) with k_norm_w
  * (either weight may be NULL = no norm), all rotated by the RoPE row rope_pos0 + s (rope NULL = no
- * rotation).  This is the layout FluxJointAttention.forward / process_attention give q and k
- * before chunking (flux_dit.py:165-171,297-301: view (B,S,3H,D), norm_q/norm_k, apply_rope).
+ * rotation; the table must hold rope_pos0 + seq rows per batch entry, which the call cannot check).  This is the
+ * layout FluxJointAttention.forward / process_attention give q and k before chunking (flux_dit.py:165-171,297-301:
+ * view (B,S,3H,D), norm_q/norm_k, apply_rope).
  */
 int dsx_rmsnorm_rope_qk(void* x, int64_t x_sb, int64_t x_ss, int32_t heads_q, int32_t heads_k,
                         const void* q_norm_w, const void* k_norm_w, float eps, const float* rope,
@@ -275,7 +277,8 @@ int dsx_rmsnorm_rope_qk(void* x, int64_t x_sb, int64_t x_ss, int32_t heads_q, in
  *   the (cos, sin) of table row (row % rows_per_batch) [+ rope_sb per batch entry] and rounded to bf16.
  * Replaces Wan's RMSNorm.forward over the full model dim (models/wan/wan_dit.py:61-78,98-99,142-143) and
  * rope_apply (wan_dit.py:54-58; the reference multiplies in complex128, this kernel in fp32).
- * x, out: (rows, D) bf16; w: (D,) bf16; rope: fp32 (pos, 64, 2) or NULL.  D % 8 == 0 (128 with rope), D <= 16384.
+ * x, out: (rows, D) bf16; w: (D,) bf16; rope: fp32 (pos, 64, 2) or NULL, rows_per_batch table rows per batch
+ * entry (not checkable here).  D % 8 == 0 (128 with rope), D <= 16384.
  * head_norm2_max (device, one float, or NULL; needs D % 128 == 0): raised (atomic maximum, never lowered) to the
  * largest squared 2-norm of a 128-wide head of an output row; the caller sets it to 0 before the first call
  * that contributes.  It is what dsx_attn_params.qk_norm2_max reads (no counterpart in the reference).
