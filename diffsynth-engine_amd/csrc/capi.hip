@@ -49,11 +49,24 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
         const u32x4 a = {r[0], r[1], r[2], r[3]}, b = {r[4 + t], r[5 + t], r[6 + t], r[7 + t]};
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
                                                          acc[t], 0, 0, 0);
-      } else {
+      } else if (KIND == 1) {
         const i32x8 a = {(int)r[0], (int)r[1], (int)r[2], (int)r[3], (int)r[4], (int)r[5], (int)r[6], (int)r[7]};
         const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
                          (int)r[15 - (t >> 1)]};
         acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
+      } else if (KIND == 2) {
+        // the 16x16 shapes: the same operand registers, a quarter of the accumulator (the first four floats)
+        const u32x4 a = {r[0], r[1], r[2], r[3]}, b = {r[4 + t], r[5 + t], r[6 + t], r[7 + t]};
+        f32x4 c = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+        acc[t][0] = c[0]; acc[t][1] = c[1]; acc[t][2] = c[2]; acc[t][3] = c[3];
+      } else {
+        const i32x8 a = {(int)r[0], (int)r[1], (int)r[2], (int)r[3], (int)r[4], (int)r[5], (int)r[6], (int)r[7]};
+        const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
+                         (int)r[15 - (t >> 1)]};
+        f32x4 c = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+        acc[t][0] = c[0]; acc[t][1] = c[1]; acc[t][2] = c[2]; acc[t][3] = c[3];
       }
     }
   }
@@ -69,14 +82,16 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
 extern "C" int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_t iters, int32_t workgroups,
                                       void* sink, int64_t* flops_out, void* stream) {
   if (!operand_bits || !sink) return DSX_ENULL;
-  if ((kind != 0 && kind != 1) || iters <= 0 || iters > (1ll << 32) || workgroups <= 0 || workgroups > (1 << 20))
+  if (kind < 0 || kind > 3 || iters <= 0 || iters > (1ll << 32) || workgroups <= 0 || workgroups > (1 << 20))
     return DSX_EBADSHAPE;
   if ((uintptr_t)operand_bits & 3) return DSX_EALIGN;
   const dim3 grid((unsigned)workgroups), block(256);
-  if (kind == 0)
-    dsx::mfma_ceiling_kernel<0><<<grid, block, 0, (hipStream_t)stream>>>((const uint32_t*)operand_bits, iters, (float*)sink);
-  else
-    dsx::mfma_ceiling_kernel<1><<<grid, block, 0, (hipStream_t)stream>>>((const uint32_t*)operand_bits, iters, (float*)sink);
-  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * 4 * (kind == 0 ? 2ll * 32 * 32 * 16 : 2ll * 32 * 32 * 64);
+  hipStream_t st = (hipStream_t)stream;
+  if (kind == 0) dsx::mfma_ceiling_kernel<0><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+  else if (kind == 1) dsx::mfma_ceiling_kernel<1><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+  else if (kind == 2) dsx::mfma_ceiling_kernel<2><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+  else dsx::mfma_ceiling_kernel<3><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+  const int64_t flops_per_mfma[4] = {2ll * 32 * 32 * 16, 2ll * 32 * 32 * 64, 2ll * 16 * 16 * 32, 2ll * 16 * 16 * 128};
+  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * 4 * flops_per_mfma[kind];
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
