@@ -340,11 +340,14 @@ def mfma_ceiling(torch, dev):
     out = {}
     g = torch.Generator(device=dev).manual_seed(0)
     for kind, name, iters in ((0, "bf16_32x32x16", 40000), (1, "fp8_32x32x64", 20000), (2, "bf16_16x16x32", 80000),
-                              (3, "fp8_16x16x128", 40000)):
+                              (3, "fp8_16x16x128", 40000), (4, "bf16_32x32x16_both_operands_change", 40000),
+                              (5, "fp8_32x32x64_both_operands_change", 20000),
+                              (6, "bf16_16x16x32_both_operands_change", 80000),
+                              (7, "fp8_16x16x128_both_operands_change", 40000)):
         for fill in ("zero", "random"):
             if fill == "zero":
                 bits = torch.zeros(16 * 256, dtype=torch.int32, device=dev)
-            elif kind in (0, 2):  # random finite bf16 pairs / e4m3 quadruples (no NaN patterns)
+            elif kind & 1 == 0:  # random finite bf16 pairs / e4m3 quadruples (no NaN patterns)
                 bits = torch.randn(16 * 256 * 2, generator=g, device=dev).bfloat16().view(torch.int32)
             else:
                 bits = torch.randn(16 * 256 * 4, generator=g, device=dev).to(torch.float8_e4m3fn).view(torch.int32)

@@ -30,7 +30,7 @@ extern "C" int dsx_check_device(void) {
 // What the chip sustains with nothing but matrix instructions in flight, for the operand bits the caller supplies
 // (all-zero operands run at the full clock; random bits draw more power and the clock management lowers the clock).
 namespace dsx {
-template <int KIND>
+template <int KIND, bool ROT = false>
 __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __restrict__ bits, int64_t iters,
                                                            float* __restrict__ sink) {
   // eight operand dwords per lane (bf16: 4 + 4 are used; fp8: 8 + 8), the same for every workgroup
@@ -45,23 +45,27 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
   for (int64_t it = 0; it < iters; ++it) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {  // four independent accumulators
+      constexpr int kA = 0;
+      const int ra = ROT ? t : kA;  // ROT: the first operand changes from one MFMA to the next as well
       if (KIND == 0) {
-        const u32x4 a = {r[0], r[1], r[2], r[3]}, b = {r[4 + t], r[5 + t], r[6 + t], r[7 + t]};
+        const u32x4 a = {r[ra], r[ra + 1], r[ra + 2], r[ra + 3]}, b = {r[8 + t], r[9 + t], r[10 + t], r[11 + t]};
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
                                                          acc[t], 0, 0, 0);
       } else if (KIND == 1) {
-        const i32x8 a = {(int)r[0], (int)r[1], (int)r[2], (int)r[3], (int)r[4], (int)r[5], (int)r[6], (int)r[7]};
+        const i32x8 a = {(int)r[ra], (int)r[ra + 1], (int)r[ra + 2], (int)r[ra + 3], (int)r[ra + 4], (int)r[ra + 5],
+                         (int)r[ra + 6], (int)r[ra + 7]};
         const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
                          (int)r[15 - (t >> 1)]};
         acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
       } else if (KIND == 2) {
         // the 16x16 shapes: the same operand registers, a quarter of the accumulator (the first four floats)
-        const u32x4 a = {r[0], r[1], r[2], r[3]}, b = {r[4 + t], r[5 + t], r[6 + t], r[7 + t]};
+        const u32x4 a = {r[ra], r[ra + 1], r[ra + 2], r[ra + 3]}, b = {r[8 + t], r[9 + t], r[10 + t], r[11 + t]};
         f32x4 c = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
         c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
         acc[t][0] = c[0]; acc[t][1] = c[1]; acc[t][2] = c[2]; acc[t][3] = c[3];
       } else {
-        const i32x8 a = {(int)r[0], (int)r[1], (int)r[2], (int)r[3], (int)r[4], (int)r[5], (int)r[6], (int)r[7]};
+        const i32x8 a = {(int)r[ra], (int)r[ra + 1], (int)r[ra + 2], (int)r[ra + 3], (int)r[ra + 4], (int)r[ra + 5],
+                         (int)r[ra + 6], (int)r[ra + 7]};
         const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
                          (int)r[15 - (t >> 1)]};
         f32x4 c = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
@@ -82,16 +86,24 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
 extern "C" int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_t iters, int32_t workgroups,
                                       void* sink, int64_t* flops_out, void* stream) {
   if (!operand_bits || !sink) return DSX_ENULL;
-  if (kind < 0 || kind > 3 || iters <= 0 || iters > (1ll << 32) || workgroups <= 0 || workgroups > (1 << 20))
+  if (kind < 0 || kind > 7 || iters <= 0 || iters > (1ll << 32) || workgroups <= 0 || workgroups > (1 << 20))
     return DSX_EBADSHAPE;
   if ((uintptr_t)operand_bits & 3) return DSX_EALIGN;
   const dim3 grid((unsigned)workgroups), block(256);
   hipStream_t st = (hipStream_t)stream;
-  if (kind == 0) dsx::mfma_ceiling_kernel<0><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
-  else if (kind == 1) dsx::mfma_ceiling_kernel<1><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
-  else if (kind == 2) dsx::mfma_ceiling_kernel<2><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
-  else dsx::mfma_ceiling_kernel<3><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink);
+#define DSX_PROBE(K, R) dsx::mfma_ceiling_kernel<K, R><<<grid, block, 0, st>>>((const uint32_t*)operand_bits, iters, (float*)sink)
+  switch (kind) {
+    case 0: DSX_PROBE(0, false); break;
+    case 1: DSX_PROBE(1, false); break;
+    case 2: DSX_PROBE(2, false); break;
+    case 3: DSX_PROBE(3, false); break;
+    case 4: DSX_PROBE(0, true); break;
+    case 5: DSX_PROBE(1, true); break;
+    case 6: DSX_PROBE(2, true); break;
+    default: DSX_PROBE(3, true); break;
+  }
+#undef DSX_PROBE
   const int64_t flops_per_mfma[4] = {2ll * 32 * 32 * 16, 2ll * 32 * 32 * 64, 2ll * 16 * 16 * 32, 2ll * 16 * 16 * 128};
-  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * 4 * flops_per_mfma[kind];
+  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * 4 * flops_per_mfma[kind & 3];
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
