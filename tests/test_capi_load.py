@@ -209,6 +209,34 @@ def test_attention_refuses_what_its_kernels_would_mis_address():
         _lib.check(_lib.DSX_EWORKSPACE, "x")
 
 
+def test_device_side_score_bound_and_head_norm_guards():
+    """qk_norm2_max describes q and k as given, so it is refused together with any fused pre-processing (before the
+    scratch question is even asked) and when misaligned; head_norm2_max needs rows made of whole 128-wide heads; the
+    probe knows eight kinds."""
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(1 << 16)
+    P, p16 = _host_attn_params(buf)
+    P.qk_norm2_max = p16 + 2
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EALIGN
+    P.qk_norm2_max = p16
+    P.q_norm_w[0] = p16
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE
+    P, p16 = _host_attn_params(buf)
+    P.qk_norm2_max, P.rope, P.rope_rows = p16, p16, 64
+    assert lib.dsx_attn_fwd(P, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_attn_fwd_static(P, None) == _lib.DSX_EBADSHAPE
+    # dsx_rmsnorm_rows(x, ldx, w, eps, rope, rope_sb, rows_per_batch, out, ldo, rows, D, head_norm2_max, stream)
+    assert lib.dsx_rmsnorm_rows(p16, 192, p16, 1e-6, None, 0, 4, p16, 192, 4, 192, p16, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_rmsnorm_rows(p16, 256, p16, 1e-6, None, 0, 4, p16, 256, 4, 256, p16 + 2, None) == _lib.DSX_EALIGN
+    assert lib.dsx_rmsnorm_rows(p16, 256, p16, 1e-6, None, 0, 4, p16, 256, 0, 256, p16, None) == _lib.DSX_OK  # no rows
+    for kind in (-1, 8):
+        assert lib.dsx_mfma_ceiling_probe(kind, p16, 1, 1, p16, None, None) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_mfma_ceiling_probe(7, None, 1, 1, p16, None, None) == _lib.DSX_ENULL
+    assert lib.dsx_gelu_erf(p16, 12, p16, 12, None, 0, None, 4, 12, None) == _lib.DSX_EBADSHAPE  # D % 8
+
+
 def test_gemm_refuses_leading_dimensions_beyond_its_32_bit_tile_offsets():
     from diffsynth_engine_amd import _lib
 
