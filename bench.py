@@ -186,8 +186,8 @@ def run_wan(torch, dev, layers, steps, warmup, with_cpu_baseline):
                                "32760 video tokens (21x60x104 latent) + 512 text tokens, batch 1, random init" % L},
         # dominant kernel: attn_plain_kernel (53 % of the step's flops); self- and cross-attention launches together
         "roofline": {"bound": "mfma", "achieved": round(attn_flops / attn_secs / 1e12, 1), "peak": PEAK_BF16 / 1e12,
-                     "unit": "TFLOP/s", "frac": round(attn_flops / attn_secs / PEAK_BF16, 4), "traffic": None,
-                     "kernel": "attn_plain_kernel", "launches": n_attn,
+                     "unit": "TFLOP/s", "frac": round(attn_flops / attn_secs / PEAK_BF16, 4),
+                     "traffic": WAN_ATTN_TRAFFIC_BYTES, "kernel": "attn_plain_kernel", "launches": n_attn,
                      "avg_launch_us": round(attn_secs / max(n_attn, 1) * 1e6, 1)},
         "detail": {"fp8_gemm_in_step": {"launches": n_gemm, "tflops": round(gemm_flops / gemm_secs / 1e12, 1),
                                         "frac_fp8_peak": round(gemm_flops / gemm_secs / PEAK_FP8, 4),
@@ -583,6 +583,10 @@ def wan_cpu_baseline(cfg, S_full, S_sample=2048, reps=2):
 # counts half the copied bytes, WRITE_SIZE all of them); profiles/flux_step_hbm_traffic_pmc.txt holds the
 # per-shape figures.
 GEMM_TRAFFIC_BYTES = 468.8e6
+# L2-miss bytes per attention call of the Wan step, averaged over its self- and cross-attention calls (one of each
+# per layer): FETCH_SIZE + WRITE_SIZE runs of `--workload wan14b --wan-layers 2 --calibrate-copy`, scaled the same
+# way (profiles/wan14b_attention_hbm_traffic_pmc.txt: self-attention 3035 + 335 MB, cross-attention 363 + 336 MB).
+WAN_ATTN_TRAFFIC_BYTES = 2034.7e6
 
 
 def main():
@@ -616,6 +620,12 @@ def main():
         sys.exit("bench.py: " + _lib.strerror(rc))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.workload == "wan14b":
         print(json.dumps(run_wan(torch, dev, args.wan_layers, args.steps, args.warmup, not args.no_cpu_baseline)))
         return
@@ -631,12 +641,6 @@ def main():
         guidance=torch.tensor([3.5], device=dev),
         text_ids=torch.zeros(1, N_TXT, 3, device=dev),
     )
-    if args.calibrate_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
     for _ in range(args.warmup):
         out = runner(**inp)
     torch.cuda.synchronize()
