@@ -195,8 +195,12 @@ class WanDiTRunner:
         ctx_q = self.quantise_context(ctx)
         for i in range(cfg["num_layers"]):
             hs = self.block(i, hs, ctx, t_mod, rope, ctx_q)
-        shift, scale = (self.vec["head.modulation"] + t).chunk(2, dim=1)  # Head.forward (wan_dit.py:234-237)
-        hq, hsc = self._modulate_q(hs, scale.reshape(B, d), shift.reshape(B, d))
+        # Head.forward (wan_dit.py:234-237).  The reference adds the (B, d) embedding to the (1, 2, d) table as it
+        # stands, so a batch of two (its batched classifier-free guidance, pipelines/wan_video.py:233-248, where both
+        # entries carry the same timestep) gets ONE (shift, scale) pair, shift from entry 0 and scale from entry 1;
+        # the same expression is evaluated here and shared by the batch (larger batches do not broadcast there either).
+        shift, scale = (self.vec["head.modulation"] + t).chunk(2, dim=1)
+        hq, hsc = self._modulate_q(hs, scale.reshape(1, d).expand(B, d), shift.reshape(1, d).expand(B, d))
         out = self.lin["head.head"](hq.view(-1, d), hsc)
         c = cfg["out_dim"]
         return out.view(B, f, h, w, pf, ph, pw, c).permute(0, 7, 1, 4, 2, 5, 3, 6).reshape(B, c, f * pf, h * ph, w * pw)

@@ -230,3 +230,25 @@ def test_i2v_small_model_step(dev):
         R(x.to(dev), ctx.to(dev), t.to(dev))  # an image-to-video checkpoint needs its image inputs
     with pytest.raises(ValueError):
         R(x.to(dev), ctx.to(dev), t.to(dev), clip_feature=clip[:, :100].to(dev), y=y.to(dev))
+
+
+def test_batch_of_two_equals_two_single_runs(dev):
+    """The pipeline's batched classifier-free guidance (pipelines/wan_video.py:233-248): latents, context and
+    timestep of the positive and the negative prompt as one batch of two.  Every row of every kernel depends on its
+    own batch entry only (modulation, gates, context), so the batch gives bit for bit what two single runs give;
+    and it matches the oracle, which evaluates the reference's expressions on the batch."""
+    from diffsynth_engine_amd.wan_dit import WanDiTRunner
+
+    cfg, sd = _small()
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(2, 16, 2, 12, 16, generator=g).bfloat16()
+    ctx = torch.randn(2, 32, 4096, generator=g).bfloat16()
+    t = torch.tensor([431.0, 431.0]).bfloat16()
+    R = WanDiTRunner(sd, cfg, scaled=True, device=dev)
+    both = R(x.to(dev), ctx.to(dev), t.to(dev))
+    for b in range(2):
+        one = R(x[b:b + 1].to(dev), ctx[b:b + 1].to(dev), t[b:b + 1].to(dev))
+        assert torch.equal(both[b:b + 1], one), b
+    assert not torch.equal(both[0], both[1])
+    want = ow.wan_dit_forward(ow.Params(sd, "fp8_scaled"), x, ctx, t, cfg)
+    assert _cos(both, want) >= 0.99
