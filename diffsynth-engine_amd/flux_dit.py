@@ -378,7 +378,11 @@ class FluxDiTRunner:
 
     # ------------------------------------------------------------------ step
     @torch.no_grad()
-    def forward(self, hidden_states, timestep, prompt_emb, pooled_prompt_emb, guidance, text_ids, image_ids=None):
+    def forward(self, hidden_states, timestep, prompt_emb, pooled_prompt_emb, guidance, text_ids, image_ids=None,
+                use_gradient_checkpointing=False, **kwargs):
+        """FluxDiT.forward's signature (flux_dit.py:392-402); the trailing arguments concern training and are ignored.
+        text_ids / image_ids / guidance may have batch 1 beside a larger batch of latents (the pipeline's batched
+        classifier-free guidance, pipelines/flux_image.py:389-399): they broadcast."""
         dev = self.device
         bf = torch.bfloat16
         B, C, Hh, Ww = hidden_states.shape
@@ -386,7 +390,7 @@ class FluxDiTRunner:
             image_ids = torch.zeros(Hh // 2, Ww // 2, 3, device=dev)
             image_ids[..., 1] += torch.arange(Hh // 2, device=dev)[:, None]
             image_ids[..., 2] += torch.arange(Ww // 2, device=dev)[None, :]
-            image_ids = image_ids.reshape(1, -1, 3).repeat(B, 1, 1)
+            image_ids = image_ids.reshape(1, -1, 3).repeat(text_ids.shape[0], 1, 1)
         cond = self._timestep_mlp("time_embedder", timestep)
         if self.has_guidance and guidance is not None:
             cond = cond + self._timestep_mlp("guidance_embedder", guidance * 1000)

@@ -186,6 +186,14 @@ def test_batch_of_two_equals_two_single_runs(dev):
     out = R(**both).cpu()
     assert torch.equal(out[0:1], R(**a).cpu())
     assert torch.equal(out[1:2], R(**b).cpu())
+    # the pipeline's own batched call (flux_image.py:389-399): latents, timestep and prompt embeddings are doubled,
+    # image_ids, text_ids and guidance stay at batch 1 and broadcast (one RoPE table for both entries); extra keyword
+    # arguments of FluxDiT.forward (flux_dit.py:400-401) are accepted
+    c = dict(a, prompt_emb=b["prompt_emb"], pooled_prompt_emb=b["pooled_prompt_emb"])
+    cfg = {k: torch.cat([a[k], c[k]], dim=0) for k in ("hidden_states", "timestep", "prompt_emb", "pooled_prompt_emb")}
+    cfg.update(guidance=a["guidance"], text_ids=a["text_ids"][:1])
+    out = R(**cfg, image_ids=None, use_gradient_checkpointing=False).cpu()
+    assert torch.equal(out[0:1], R(**a).cpu()) and torch.equal(out[1:2], R(**c).cpu())
 
 
 def test_three_step_denoising_loop(dev):
