@@ -252,3 +252,23 @@ def test_batch_of_two_equals_two_single_runs(dev):
     assert not torch.equal(both[0], both[1])
     want = ow.wan_dit_forward(ow.Params(sd, "fp8_scaled"), x, ctx, t, cfg)
     assert _cos(both, want) >= 0.99
+
+
+def test_i2v_batch_of_two_equals_two_single_runs(dev):
+    """The same batched guidance call for the image-to-video form: clip_feature and y are doubled with the latents
+    (pipelines/wan_video.py:237-240)."""
+    from diffsynth_engine_amd.wan_dit import WanDiTRunner
+
+    cfg, sd = _small_i2v()
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(2, 16, 2, 12, 16, generator=g).bfloat16()
+    y = torch.randn(1, 16, 2, 12, 16, generator=g).bfloat16().repeat(2, 1, 1, 1, 1)
+    ctx = torch.randn(2, 24, 4096, generator=g).bfloat16()
+    clip = torch.randn(1, 257, 256, generator=g).bfloat16().repeat(2, 1, 1)
+    t = torch.tensor([610.0, 610.0]).bfloat16()
+    R = WanDiTRunner(sd, cfg, scaled=True, device=dev)
+    both = R(x=x.to(dev), context=ctx.to(dev), timestep=t.to(dev), clip_feature=clip.to(dev), y=y.to(dev))
+    for b in range(2):
+        one = R(x=x[b:b + 1].to(dev), context=ctx[b:b + 1].to(dev), timestep=t[b:b + 1].to(dev),
+                clip_feature=clip[b:b + 1].to(dev), y=y[b:b + 1].to(dev))
+        assert torch.equal(both[b:b + 1], one), b
