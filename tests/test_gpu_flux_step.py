@@ -46,6 +46,34 @@ def test_two_block_step_matches_cpu_oracle(dev, mode, scaled):
     assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
 
 
+def test_non_square_latent_matches_oracle(dev):
+    """A 24 x 40 latent (12 x 20 = 240 image tokens): rows and columns of the patch grid, of the image ids and of
+    the unpatchify are different numbers, so a swapped pair shows.  Oracle on the CPU (its patchify, prepare_image_ids
+    and unpatchify are pinned to the reference's vectors); also with the ids passed explicitly, as the pipeline does
+    (pipelines/flux_image.py:352-358)."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=31, bias_std=0.02)
+    g = torch.Generator().manual_seed(32)
+    inp = dict(hidden_states=torch.randn(1, 16, 24, 40, generator=g).bfloat16(), timestep=torch.tensor([700.0]),
+               prompt_emb=torch.randn(1, 24, 4096, generator=g).bfloat16(),
+               pooled_prompt_emb=torch.randn(1, 768, generator=g).bfloat16(), guidance=torch.tensor([3.5]),
+               text_ids=torch.zeros(1, 24, 3))
+    want = oflux.flux_dit_forward(oflux.Params(sd, "fp8_scaled"), **inp, num_double=1, num_single=1)
+    R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    inp_dev = {k: v.to(dev) for k, v in inp.items()}
+    got = R(**inp_dev)
+    assert got.shape == (1, 16, 24, 40)
+    assert _cos(got, want) >= 0.995, _cos(got, want)
+    ids = torch.zeros(12, 20, 3)
+    ids[..., 1] += torch.arange(12)[:, None]
+    ids[..., 2] += torch.arange(20)[None, :]
+    assert torch.equal(R(**inp_dev, image_ids=ids.reshape(1, 240, 3).to(dev)), got)
+    # the transposed grid (ids of a 20 x 12 image) is a different RoPE table and a visibly different output
+    wrong = R(**inp_dev, image_ids=ids.transpose(0, 1).reshape(1, 240, 3).to(dev))
+    assert _cos(wrong, want) < _cos(got, want) - 1e-3
+
+
 def test_deeper_step_matches_oracle(dev):
     """4 double + 6 single blocks at 32x32 latent (256 image + 64 text tokens), oracle on the CPU."""
     from diffsynth_engine_amd.flux_dit import FluxDiTRunner
