@@ -74,6 +74,28 @@ def test_non_square_latent_matches_oracle(dev):
     assert _cos(wrong, want) < _cos(got, want) - 1e-3
 
 
+def test_checkpoint_without_guidance_embedder(dev):
+    """FluxDiT(disable_guidance_embedder=True) (flux_dit.py:341-347,412-414): no guidance_embedder.* entries in the
+    checkpoint, and the guidance argument, whatever it holds, does not enter the conditioning."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=41, bias_std=0.02, guidance=False)
+    assert not any(k.startswith("guidance_embedder") for k in sd)
+    inp = _inputs(16, 24, seed=42)
+    want = oflux.flux_dit_forward(oflux.Params(sd, "fp8_scaled"), **inp, num_double=1, num_single=1)
+    R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    assert not R.has_guidance
+    inp_dev = {k: v.to(dev) for k, v in inp.items()}
+    got = R(**inp_dev)
+    assert _cos(got, want) >= 0.995, _cos(got, want)
+    assert torch.equal(R(**dict(inp_dev, guidance=None)), got)
+    assert torch.equal(R(**dict(inp_dev, guidance=torch.tensor([9.0], device=dev))), got)
+    # with the embedder the guidance value does matter
+    sd_g = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=41, bias_std=0.02, guidance=True)
+    Rg = FluxDiTRunner(sd_g, 1, 1, scaled=True, device=dev)
+    assert not torch.equal(Rg(**inp_dev), Rg(**dict(inp_dev, guidance=torch.tensor([9.0], device=dev))))
+
+
 def test_deeper_step_matches_oracle(dev):
     """4 double + 6 single blocks at 32x32 latent (256 image + 64 text tokens), oracle on the CPU."""
     from diffsynth_engine_amd.flux_dit import FluxDiTRunner
