@@ -46,7 +46,8 @@ def test_two_block_step_matches_cpu_oracle(dev, mode, scaled):
     assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
 
 
-def test_non_square_latent_matches_oracle(dev):
+@pytest.mark.parametrize("n_txt", [24, 77])
+def test_non_square_latent_matches_oracle(dev, n_txt):
     """A 24 x 40 latent (12 x 20 = 240 image tokens): rows and columns of the patch grid, of the image ids and of
     the unpatchify are different numbers, so a swapped pair shows.  Oracle on the CPU (its patchify, prepare_image_ids
     and unpatchify are pinned to the reference's vectors); also with the ids passed explicitly, as the pipeline does
@@ -56,9 +57,9 @@ def test_non_square_latent_matches_oracle(dev):
     sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=31, bias_std=0.02)
     g = torch.Generator().manual_seed(32)
     inp = dict(hidden_states=torch.randn(1, 16, 24, 40, generator=g).bfloat16(), timestep=torch.tensor([700.0]),
-               prompt_emb=torch.randn(1, 24, 4096, generator=g).bfloat16(),
+               prompt_emb=torch.randn(1, n_txt, 4096, generator=g).bfloat16(),
                pooled_prompt_emb=torch.randn(1, 768, generator=g).bfloat16(), guidance=torch.tensor([3.5]),
-               text_ids=torch.zeros(1, 24, 3))
+               text_ids=torch.zeros(1, n_txt, 3))  # (77 text tokens: a text segment that no tile size divides)
     want = oflux.flux_dit_forward(oflux.Params(sd, "fp8_scaled"), **inp, num_double=1, num_single=1)
     R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
     inp_dev = {k: v.to(dev) for k, v in inp.items()}
