@@ -46,7 +46,7 @@ def test_two_block_step_matches_cpu_oracle(dev, mode, scaled):
     assert _cos(got, want) >= _floor(want, want_dev), (_cos(got, want), _cos(want, want_dev))
 
 
-@pytest.mark.parametrize("n_txt", [24, 77])
+@pytest.mark.parametrize("n_txt", [24, 77, 4])
 def test_non_square_latent_matches_oracle(dev, n_txt):
     """A 24 x 40 latent (12 x 20 = 240 image tokens): rows and columns of the patch grid, of the image ids and of
     the unpatchify are different numbers, so a swapped pair shows.  Oracle on the CPU (its patchify, prepare_image_ids
