@@ -144,12 +144,24 @@ def ingest_state_dict(state_dict, device, scaled: bool, as_linear=None):
     return lin, other
 
 
+def count_blocks(names, prefix: str) -> int:
+    """1 + the largest index i among names of the form ``<prefix><i>.…`` (0 if there is none)."""
+    n = 0
+    for name in names:
+        if name.startswith(prefix):
+            head = name[len(prefix):].split(".", 1)[0]
+            if head.isdigit():
+                n = max(n, int(head) + 1)
+    return n
+
+
 class FluxDiTRunner:
     """Holds quantised weights of a Flux-architecture DiT and runs one denoising step.  The hidden size comes
     from the checkpoint (``x_embedder.weight``); heads are 128 wide (``heads`` = hidden / 128 unless given)."""
 
-    def __init__(self, state_dict, num_double: int = 19, num_single: int = 38, scaled: bool = True,
-                 device="cuda:0", heads: Optional[int] = None, axes_dim=AXES_DIM, qk_prep: str = "gemm"):
+    def __init__(self, state_dict, num_double: Optional[int] = None, num_single: Optional[int] = None,
+                 scaled: bool = True, device="cuda:0", heads: Optional[int] = None, axes_dim=AXES_DIM,
+                 qk_prep: str = "gemm"):
         self.device = torch.device(device)
         self.scaled = scaled
         # Where the per-head RMSNorm and the RoPE rotation of q and k happen (flux_dit.py:165-171,179-180,297-301):
@@ -159,8 +171,13 @@ class FluxDiTRunner:
         if qk_prep not in ("gemm", "attention"):
             raise ValueError("qk_prep must be 'gemm' or 'attention', got %r" % (qk_prep,))
         self.qk_prep = qk_prep
-        self.num_double, self.num_single = num_double, num_single
         self.lin, other = ingest_state_dict(state_dict, self.device, scaled)
+        # block counts: given, or as many as the checkpoint holds (FluxDiT builds 19 + 38, flux_dit.py:352-356)
+        if num_double is None:
+            num_double = count_blocks(self.lin, "blocks.")
+        if num_single is None:
+            num_single = count_blocks(self.lin, "single_blocks.")
+        self.num_double, self.num_single = num_double, num_single
         self.norm_w: Dict[str, torch.Tensor] = {}
         for key, t in other.items():
             if key.endswith(".weight") and t.dim() == 1:

@@ -19,33 +19,55 @@ The reference wires FP8 for Flux only (models/flux/flux_dit.py:404; pipelines/ba
 rest); here every Linear of the Wan DiT runs through the same scaled e4m3 GEMM as Flux.
 """
 import math
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
 from . import ops
-from .flux_dit import _Linear, _gemm_pair, ingest_state_dict
+from .flux_dit import _Linear, _gemm_pair, count_blocks, ingest_state_dict
 
 
 IMAGE_ROWS = 257  # CLIP tokens in front of the text context (the split is hard-coded, wan_dit.py:138-139)
 
 
+def wan_config_from_shapes(shapes: Dict[str, tuple], eps: float = 1e-6) -> dict:
+    """The constructor arguments of WanDiT (wan_dit.py:247-262; conf/models/wan/dit/*.json) that the runner needs,
+    read off a checkpoint's tensor shapes: ``shapes`` maps state-dict names to shapes.  Heads are 128 wide (the
+    attention kernel's head width: 40 heads at dim 5120, 12 at 1536, as in the reference's configurations); eps
+    is not in a checkpoint (1e-6 in every configuration the reference ships)."""
+    conv = tuple(shapes["patch_embedding.weight"])  # (dim, in_dim, pf, ph, pw)
+    if len(conv) != 5:
+        raise ValueError("patch_embedding.weight must be the 5-D Conv3d weight, got shape %s" % (conv,))
+    dim, patch = conv[0], tuple(conv[2:])
+    if dim % 128:
+        raise ValueError("WanDiTRunner needs dim = heads * 128, got dim %d" % dim)
+    layers = count_blocks((k for k in shapes if k.endswith(".weight")), "blocks.")
+    out_features = shapes["head.head.weight"][0]
+    return {"dim": dim, "in_dim": conv[1], "ffn_dim": shapes["blocks.0.ffn.0.weight"][0],
+            "out_dim": out_features // math.prod(patch), "text_dim": shapes["text_embedding.0.weight"][1],
+            "freq_dim": shapes["time_embedding.0.weight"][1], "eps": eps, "patch_size": patch,
+            "num_heads": dim // 128, "num_layers": layers,
+            "has_image_input": "img_emb.proj.1.weight" in shapes}
+
+
 class WanDiTRunner:
-    def __init__(self, state_dict, cfg: dict, scaled: bool = True, device="cuda:0"):
-        self.cfg = cfg
+    def __init__(self, state_dict, cfg: Optional[dict] = None, scaled: bool = True, device="cuda:0"):
         self.device = torch.device(device)
         self.scaled = scaled
         # self-attention reads the largest head norms of q and k on the device and drops the running softmax
         # maximum when they allow it (False: always the running maximum)
         self.device_score_bound = True
-        d = cfg["dim"]
+        shapes: Dict[str, tuple] = {}
 
         def conv_as_linear(key, t):  # Conv3d with kernel == stride is a Linear over each patch
-            return t.reshape(d, -1) if key == "patch_embedding.weight" else None
+            shapes[key] = tuple(t.shape)
+            return t.reshape(t.shape[0], -1) if key == "patch_embedding.weight" else None
 
         # key order does not matter: biases are attached once every weight is known; what is not a Linear
         # (modulation vectors, norm weights and the affine bias of norm3) lands in `vec` under its full key
         self.lin, self.vec = ingest_state_dict(state_dict, self.device, scaled, as_linear=conv_as_linear)
+        # dims: given (the reference's conf/models/wan/dit/*.json), or read off the checkpoint's shapes
+        self.cfg = dict(wan_config_from_shapes(shapes) if cfg is None else cfg)
         self.has_image_input = "img_emb.proj.1" in self.lin
 
     # ------------------------------------------------------------------ helpers

@@ -66,3 +66,27 @@ def test_flux_runner_refuses_entries_it_has_no_use_for():
     sd = _tiny()
     with pytest.raises(KeyError, match="modulation|norm3"):
         FluxDiTRunner(sd, 0, 0, scaled=True, device="cpu")
+
+
+def test_wan_dims_and_flux_block_counts_are_read_off_a_checkpoint():
+    """WanDiT's constructor arguments (wan_dit.py:247-262, conf/models/wan/dit/*.json) from tensor shapes alone
+    (reduced widths; text-to-video twice and the image-to-video form); Flux block counts from the key names."""
+    from diffsynth_engine_amd.flux_dit import count_blocks
+    from diffsynth_engine_amd.wan_dit import wan_config_from_shapes
+    from oracle import wan as ow
+
+    base = ow.config_14b()
+    for cfg, clip in ((dict(base, dim=256, ffn_dim=640, num_heads=2, num_layers=3), None),
+                      (dict(base, dim=384, ffn_dim=512, num_heads=3, num_layers=2, out_dim=8, freq_dim=64, text_dim=96), None),
+                      (dict(base, dim=128, ffn_dim=256, num_heads=1, num_layers=2, in_dim=36, patch_size=(1, 2, 2)), 80)):
+        small = cfg
+        sd = ow.init_params(small, dtype=torch.bfloat16, seed=0, **({"clip_dim": clip} if clip else {}))
+        got = wan_config_from_shapes({k: tuple(v.shape) for k, v in sd.items()})
+        for key in ("dim", "in_dim", "ffn_dim", "out_dim", "text_dim", "freq_dim", "eps", "num_heads", "num_layers"):
+            assert got[key] == small[key], (key, got[key], small[key])
+        assert tuple(got["patch_size"]) == tuple(small["patch_size"]) and got["has_image_input"] == bool(clip)
+    names = ["blocks.0.attn.a_to_qkv", "blocks.18.ff_a.0", "single_blocks.37.proj_out", "single_blocks.4.norm.linear", "x_embedder"]
+    assert (count_blocks(names, "blocks."), count_blocks(names, "single_blocks.")) == (19, 38)
+    assert count_blocks(["x_embedder"], "blocks.") == 0
+    with pytest.raises(ValueError):
+        wan_config_from_shapes({"patch_embedding.weight": (100, 16, 1, 2, 2)})
