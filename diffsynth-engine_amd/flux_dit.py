@@ -231,6 +231,10 @@ class FluxDiTRunner:
     def add_lora(self, name: str, down: torch.Tensor, up: torch.Tensor, coef: float = 1.0):
         """Attach an unfused LoRA (``coef`` = scale * alpha / rank) to the Linear called ``name``; the AdaLN
         projections are stacked at construction and take no LoRA here."""
+        if name in self.mod_slices:
+            raise ValueError("%s is one of the stacked AdaLN projections and takes no unfused LoRA: fuse it into the "
+                             "weight (LoRALinear.add_frozen_lora, models/basic/lora.py:108-124) before the runner "
+                             "is built" % name)
         self.lin[name].add_lora(down, up, coef)
 
     def _qk_in_gemm(self, rows, *layers) -> bool:

@@ -10,8 +10,9 @@ pipeline keeps calling ``self.dit(...)`` (pipelines/flux_image.py:513-526, pipel
 
 The runner is built from ``module.state_dict()`` (the reference's parameter names) on the module's device and keeps
 its own e4m3 copy of every Linear weight; the module's parameters stay as they are, so ``restore_forward`` gives the
-original behaviour back.  Later changes to the module's parameters (``load_state_dict``, fused LoRA) do not reach
-the runner: call ``accelerate_*`` again.
+original behaviour back.  Unfused LoRAs the module's LoRALinear layers carry at that moment are attached to the
+runner's linears; a LoRA on one of Flux's AdaLN projections has to be fused first.  Later changes to the module
+(``load_state_dict``, LoRAs added, removed, fused or rescaled) do not reach the runner: call ``accelerate_*`` again.
 """
 from typing import Optional
 
@@ -44,6 +45,26 @@ def _scaled_mode(state_dict, scaled: Optional[bool]) -> bool:
     return True
 
 
+def _state_dict(module: nn.Module):
+    """``module.state_dict()`` without the copies LoRALinear keeps of weights it has fused a LoRA into
+    (``_original_weight``, models/basic/lora.py:66,119-120): the fused ``weight`` is the one to run."""
+    return {k: v for k, v in module.state_dict().items() if not k.endswith("._original_weight")}
+
+
+def _attach_loras(module: nn.Module, runner) -> int:
+    """Unfused LoRAs of the module's LoRALinear layers (``_lora_dict``, models/basic/lora.py:63,80-100: name ->
+    LoRA with ``scale``, ``alpha``, ``rank`` and ``up`` / ``down`` as bias-free Linears or plain tensors) go to the
+    runner's linears of the same names; LoRALinear.forward adds ``scale * alpha / rank * up(down(x))`` (:29-32,137-141)."""
+    n = 0
+    for name, sub in module.named_modules():
+        for lora in getattr(sub, "_lora_dict", {}).values():
+            up = lora.up.weight if isinstance(lora.up, nn.Module) else lora.up
+            down = lora.down.weight if isinstance(lora.down, nn.Module) else lora.down
+            runner.add_lora(name, down.detach(), up.detach(), float(lora.scale) * float(lora.alpha) / float(lora.rank))
+            n += 1
+    return n
+
+
 def _rebind(module: nn.Module, runner):
     if _ORIGINAL not in module.__dict__:
         # the bound method the instance had: a class attribute normally, an instance attribute if someone
@@ -57,8 +78,9 @@ def _rebind(module: nn.Module, runner):
 def accelerate_flux_dit(dit: nn.Module, scaled: Optional[bool] = None, **runner_options) -> FluxDiTRunner:
     """``dit``: a module with FluxDiT's parameter names (flux_dit.py:338-364).  Returns the runner that now
     answers ``dit(hidden_states, timestep, prompt_emb, pooled_prompt_emb, guidance, text_ids, image_ids=None)``."""
-    sd = dit.state_dict()
+    sd = _state_dict(dit)
     runner = FluxDiTRunner(sd, scaled=_scaled_mode(sd, scaled), device=_device_of(dit), **runner_options)
+    _attach_loras(dit, runner)
     return _rebind(dit, runner)
 
 
@@ -66,8 +88,9 @@ def accelerate_wan_dit(dit: nn.Module, cfg: Optional[dict] = None, scaled: Optio
     """``dit``: a module with WanDiT's parameter names (wan_dit.py:247-299).  ``cfg``: the constructor arguments
     of conf/models/wan/dit/*.json; left out, they are read off the parameter shapes.  Returns the runner that now
     answers ``dit(x, context, timestep, clip_feature=None, y=None)``."""
-    sd = dit.state_dict()
+    sd = _state_dict(dit)
     runner = WanDiTRunner(sd, cfg, scaled=_scaled_mode(sd, scaled), device=_device_of(dit))
+    _attach_loras(dit, runner)
     return _rebind(dit, runner)
 
 

@@ -70,6 +70,11 @@ class WanDiTRunner:
         self.cfg = dict(wan_config_from_shapes(shapes) if cfg is None else cfg)
         self.has_image_input = "img_emb.proj.1" in self.lin
 
+    def add_lora(self, name: str, down: torch.Tensor, up: torch.Tensor, coef: float = 1.0):
+        """Attach an unfused LoRA (``coef`` = scale * alpha / rank, models/basic/lora.py:29-32,137-141) to the
+        Linear called ``name``."""
+        self.lin[name].add_lora(down, up, coef)
+
     # ------------------------------------------------------------------ helpers
     def _linear_bf16(self, x, name):
         shp = x.shape

@@ -106,3 +106,82 @@ def test_wan_module_runs_the_runner_with_dims_read_off_the_checkpoint(dev):
     assert torch.equal(got, dit(x=x, context=ctx, timestep=t))  # the pipeline's keyword form, wan_video.py:294-368
     restore_forward(dit)
     assert dit(x, ctx, t) == "module's own forward"
+
+
+class _LoRA:
+    """The attributes of the reference's LoRA objects that LoRALinear.forward uses (models/basic/lora.py:9-32)."""
+
+    def __init__(self, scale, rank, alpha, up, down, as_linear):
+        self.scale, self.rank, self.alpha = scale, rank, alpha
+        if as_linear:  # LoRALinear.add_lora wraps the factors in bias-free Linears (lora.py:92-99)
+            self.up, self.down = nn.Linear(up.shape[1], up.shape[0], bias=False), nn.Linear(down.shape[1], down.shape[0], bias=False)
+            self.up.weight.data, self.down.weight.data = up, down
+        else:
+            self.up, self.down = up, down
+
+
+def _give_lora(dit, name, lora):
+    sub = dit.get_submodule(name)
+    if "_lora_dict" not in sub.__dict__:
+        object.__setattr__(sub, "_lora_dict", {})
+    sub._lora_dict["lora%d" % len(sub._lora_dict)] = lora
+
+
+def test_unfused_loras_of_the_module_reach_the_runner(dev):
+    """LoRALinear.forward (lora.py:137-141): w_x + sum of scale * alpha / rank * up(down(x)) over ``_lora_dict``;
+    a weight a LoRA was fused into brings an ``_original_weight`` copy in the state dict, which must not be run."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+    from diffsynth_engine_amd.install import accelerate_flux_dit
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=7, bias_std=0.02)
+    dit = shell_from(sd, dev)
+    g = torch.Generator().manual_seed(8)
+    direct = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    for i, (name, r) in enumerate({"blocks.0.attn.a_to_qkv": 16, "blocks.0.ff_b.2": 8, "single_blocks.0.proj_out": 4}.items()):
+        n, k = sd[name + ".weight"].shape
+        down = (torch.randn(r, k, generator=g) * 0.05).bfloat16().to(dev)
+        up = (torch.randn(n, r, generator=g) * 0.05).bfloat16().to(dev)
+        _give_lora(dit, name, _LoRA(0.8, r, 2 * r, up, down, as_linear=bool(i % 2)))
+        direct.add_lora(name, down, up, 0.8 * (2 * r) / r)
+    dit.get_submodule("blocks.0.attn.a_to_out").register_buffer(
+        "_original_weight", torch.zeros_like(sd["blocks.0.attn.a_to_out.weight"]).to(dev))
+    inp = _flux_inputs(dev)
+    got = accelerate_flux_dit(dit)(**inp)
+    assert torch.equal(got, direct(**inp))
+    assert not torch.equal(got, FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)(**inp))  # the LoRAs are in there
+    # a LoRA on a stacked AdaLN projection cannot ride along unfused: loud, not dropped
+    n, k = sd["blocks.0.norm1_a.linear.weight"].shape
+    _give_lora(dit, "blocks.0.norm1_a.linear", _LoRA(1.0, 4, 4, torch.zeros(n, 4, device=dev), torch.zeros(4, k, device=dev), False))
+    with pytest.raises(ValueError):
+        accelerate_flux_dit(dit)
+
+
+def test_wan_runner_with_unfused_loras_matches_the_oracle(dev):
+    """One Wan block with low-rank pairs on a projection that feeds RMSNorm (q), on one behind a gated residual (o),
+    on a cross-attention k and on the first FFN layer, against the oracle with the same pairs."""
+    from diffsynth_engine_amd.install import accelerate_wan_dit
+
+    cfg = dict(ow.config_14b(), dim=512, ffn_dim=1024, num_heads=4, num_layers=1)
+    sd = ow.init_params(cfg, dtype=torch.bfloat16, seed=11, bias_std=0.02)
+    dit = shell_from(sd, dev)
+    P = ow.Params(sd, "fp8_scaled")
+    g = torch.Generator().manual_seed(12)
+    for name, r in {"blocks.0.self_attn.q": 16, "blocks.0.self_attn.o": 8, "blocks.0.cross_attn.k": 4, "blocks.0.ffn.0": 32}.items():
+        n, k = sd[name + ".weight"].shape
+        down = (torch.randn(r, k, generator=g) * 0.05).bfloat16()
+        up = (torch.randn(n, r, generator=g) * 0.05).bfloat16()
+        P.lora[name] = [(down, up, 0.5)]
+        _give_lora(dit, name, _LoRA(0.5, r, r, up.to(dev), down.to(dev), as_linear=True))
+    f, h, w = 2, 6, 8
+    S = f * h * w
+    x = torch.randn(1, S, 512, generator=g).bfloat16()
+    ctx = torch.randn(1, 40, 512, generator=g).bfloat16()
+    t_mod = (torch.randn(1, 6, 512, generator=g) * 0.3).bfloat16()
+    freqs = ow.freqs_cis_3d(128, f, h, w)
+    want = ow.dit_block(P, 0, x, ctx, t_mod, freqs, cfg)
+    plain = ow.dit_block(ow.Params(sd, "fp8_scaled"), 0, x, ctx, t_mod, freqs, cfg)
+    cos = lambda a, b: torch.nn.functional.cosine_similarity(a.float().flatten().cpu(), b.float().flatten().cpu(), dim=0).item()
+    assert cos(plain, want) < 0.9999  # the low-rank terms matter in this set-up
+    R = accelerate_wan_dit(dit)
+    got = R.block(0, x.to(dev), ctx.to(dev), t_mod.to(dev), R.rope_table(f, h, w))
+    assert cos(got, want) >= 0.9995, cos(got, want)
