@@ -31,6 +31,21 @@ EPS = 1e-6
 SCALE_SUFFIX = ".weight_scale"  # per-tensor scale of an already quantised weight, as enable_fp8_linear's buffer names it
 
 
+def _lora_factors(down: torch.Tensor, up: torch.Tensor, coef: float, n: int, k: int, dev):
+    """(down e4m3 (r', K), its scale, up e4m3 (N, r'), its scale x coef) with the rank zero-padded to r' % 16 == 0."""
+    if tuple(down.shape[1:]) != (k,) or up.shape[0] != n or up.shape[1] != down.shape[0]:
+        raise ValueError("LoRA factors (%s, %s) do not fit a Linear %d -> %d" % (tuple(down.shape), tuple(up.shape), k, n))
+    r = down.shape[0]
+    rp = (r + 15) // 16 * 16
+    d = torch.zeros((rp, k), dtype=torch.bfloat16, device=dev)
+    d[:r] = down.to(dev, torch.bfloat16)
+    u = torch.zeros((n, rp), dtype=torch.bfloat16, device=dev)
+    u[:, :r] = up.to(dev, torch.bfloat16)
+    dq, ds = ops.quantize_weight_fp8(d, scaled=True)
+    uq, us = ops.quantize_weight_fp8(u, scaled=True)
+    return dq, ds, uq, (us * coef).float()
+
+
 class _Linear:
     """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias, plus optional unfused LoRA pairs."""
 
@@ -51,16 +66,7 @@ class _Linear:
         """Unfused low-rank update y += coef * up(down(x)) (models/basic/lora.py:29-32,137-141); both factors are
         stored as e4m3 like every other Linear under fp8 inference.  The rank is zero-padded to a multiple of 16
         (the GEMM's K granularity) and the coefficient is folded into the up factor's scale."""
-        r = down.shape[0]
-        rp = (r + 15) // 16 * 16
-        dev = self.w.device
-        d = torch.zeros((rp, self.k), dtype=torch.bfloat16, device=dev)
-        d[:r] = down.to(dev, torch.bfloat16)
-        u = torch.zeros((self.n, rp), dtype=torch.bfloat16, device=dev)
-        u[:, :r] = up.to(dev, torch.bfloat16)
-        dq, ds = ops.quantize_weight_fp8(d, scaled=True)
-        uq, us = ops.quantize_weight_fp8(u, scaled=True)
-        self.loras.append((dq, ds, uq, (us * coef).float()))
+        self.loras.append(_lora_factors(down, up, coef, self.n, self.k, self.w.device))
 
     def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None, qk=None):
         """Keyword arguments of ``ops.fp8_gemm`` for this layer applied to ``a_q``."""
@@ -214,6 +220,7 @@ class FluxDiTRunner:
             names += [f"blocks.{i}.norm1_a.linear", f"blocks.{i}.norm1_b.linear"]
         names += [f"single_blocks.{i}.norm.linear" for i in range(self.num_single)]
         names.append("final_norm_out.linear")
+        self.mod_loras: Dict[str, list] = {}
         self.mod_slices, off = {}, 0
         ws, ss, bs = [], [], []
         one = torch.ones((), dtype=torch.float32, device=self.device)
@@ -229,12 +236,13 @@ class FluxDiTRunner:
         self.mod_bias = torch.cat(bs).contiguous()
 
     def add_lora(self, name: str, down: torch.Tensor, up: torch.Tensor, coef: float = 1.0):
-        """Attach an unfused LoRA (``coef`` = scale * alpha / rank) to the Linear called ``name``; the AdaLN
-        projections are stacked at construction and take no LoRA here."""
-        if name in self.mod_slices:
-            raise ValueError("%s is one of the stacked AdaLN projections and takes no unfused LoRA: fuse it into the "
-                             "weight (LoRALinear.add_frozen_lora, models/basic/lora.py:108-124) before the runner "
-                             "is built" % name)
+        """Attach an unfused LoRA (``coef`` = scale * alpha / rank) to the Linear called ``name``, the stacked
+        AdaLN projections included."""
+        if name in self.mod_slices:  # a slice of the stacked matrix: its low-rank terms are added per step
+            lo, hi = self.mod_slices[name]
+            self.mod_loras.setdefault(name, []).append(
+                _lora_factors(down, up, coef, hi - lo, self.mod_w.shape[1], self.device))
+            return
         self.lin[name].add_lora(down, up, coef)
 
     def _qk_in_gemm(self, rows, *layers) -> bool:
@@ -275,6 +283,12 @@ class FluxDiTRunner:
         """linear(silu(cond)) of every AdaLN layer: one pass over the stacked weights."""
         a_q, a_s = ops.quantize_fp8(torch.nn.functional.silu(cond), scaled=self.scaled)
         out = ops.fp8_gemv_rowscale(a_q, self.mod_w, a_s, self.mod_row_scale, self.mod_bias)
+        for name, loras in self.mod_loras.items():  # LoRALinear.forward: w_x += lora(x), lora.py:137-141
+            lo, hi = self.mod_slices[name]
+            piece = out[:, lo:hi]
+            for dq, ds, uq, us in loras:
+                hq, hs = ops.quantize_fp8(ops.fp8_gemm(a_q, dq, a_s, ds, None), scaled=True)
+                ops.fp8_gemm(hq, uq, hs, us, None, resid=piece, out=piece)
         return {n: out[:, lo:hi] for n, (lo, hi) in self.mod_slices.items()}
 
     def _modulate_q(self, x, scale, shift):

@@ -11,7 +11,7 @@ pipeline keeps calling ``self.dit(...)`` (pipelines/flux_image.py:513-526, pipel
 The runner is built from ``module.state_dict()`` (the reference's parameter names) on the module's device and keeps
 its own e4m3 copy of every Linear weight; the module's parameters stay as they are, so ``restore_forward`` gives the
 original behaviour back.  Unfused LoRAs the module's LoRALinear layers carry at that moment are attached to the
-runner's linears; a LoRA on one of Flux's AdaLN projections has to be fused first.  Later changes to the module
+runner's linears.  Later changes to the module
 (``load_state_dict``, LoRAs added, removed, fused or rescaled) do not reach the runner: call ``accelerate_*`` again.
 """
 from typing import Optional

@@ -291,7 +291,9 @@ def test_unfused_lora_on_runner_linears(dev):
     R = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
     g = torch.Generator().manual_seed(32)
     targets = {"blocks.0.attn.a_to_qkv": 16, "blocks.0.attn.b_to_out": 8, "blocks.0.ff_a.2": 32,
-               "single_blocks.0.to_qkv_mlp": 16, "single_blocks.0.proj_out": 4}
+               "single_blocks.0.to_qkv_mlp": 16, "single_blocks.0.proj_out": 4,
+               # AdaLN projections (the runner keeps them stacked in one matrix; M = 1 products)
+               "blocks.0.norm1_a.linear": 8, "single_blocks.0.norm.linear": 16}
     for name, r in targets.items():
         n, k = sd[name + ".weight"].shape
         down = (torch.randn(r, k, generator=g) * 0.05).bfloat16()
@@ -310,6 +312,11 @@ def test_unfused_lora_on_runner_linears(dev):
     base_a, _ = oflux.joint_block(base, 0, img, txt, cond, freqs)
     assert _cos(base_a, want_a) < 0.9999  # the low-rank terms matter in this set-up
     mods = R._modulations(cond.to(dev))
+    for name in ("blocks.0.norm1_a.linear", "blocks.0.norm1_b.linear", "single_blocks.0.norm.linear"):
+        silu = torch.nn.functional.silu(cond)
+        assert _cos(mods[name], P.linear(silu, name)) >= 0.9995, name
+        if name in targets:  # and the low-rank term is what makes it so
+            assert _cos(mods[name], base.linear(silu, name)) < 0.999, name
     got_a, got_b = R._joint_block(0, img.to(dev), txt.to(dev), mods["blocks.0.norm1_a.linear"],
                                   mods["blocks.0.norm1_b.linear"], rope)
     assert _cos(got_a, want_a) >= 0.9995 and _cos(got_b, want_b) >= 0.9995, (_cos(got_a, want_a), _cos(got_b, want_b))

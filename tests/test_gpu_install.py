@@ -149,9 +149,9 @@ def test_unfused_loras_of_the_module_reach_the_runner(dev):
     got = accelerate_flux_dit(dit)(**inp)
     assert torch.equal(got, direct(**inp))
     assert not torch.equal(got, FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)(**inp))  # the LoRAs are in there
-    # a LoRA on a stacked AdaLN projection cannot ride along unfused: loud, not dropped
+    # factors that do not fit their Linear are refused, not run
     n, k = sd["blocks.0.norm1_a.linear.weight"].shape
-    _give_lora(dit, "blocks.0.norm1_a.linear", _LoRA(1.0, 4, 4, torch.zeros(n, 4, device=dev), torch.zeros(4, k, device=dev), False))
+    _give_lora(dit, "blocks.0.norm1_a.linear", _LoRA(1.0, 4, 4, torch.zeros(n, 4, device=dev), torch.zeros(4, k + 16, device=dev), False))
     with pytest.raises(ValueError):
         accelerate_flux_dit(dit)
 
