@@ -17,6 +17,9 @@
 // reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
 // One launch can carry two independent problems (the image- and text-stream linears of a joint
 // block): their tiles share the grid, so the small problem runs on CUs the large one leaves idle.
+// A launch with at most 128 such tiles (half the compute units) runs the same kernel with four waves as
+// 2x2 on tiles of 256 (n) x 128 (m) instead: twice as many workgroups, same wave tile, same K order,
+// same bits.
 #include "attn_internal.h"
 #include "common.h"
 
@@ -354,8 +357,14 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
   }
 }
 
-template <bool RESID, bool QK>
-__global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
+// s_waitcnt immediate for vmcnt(vm) and lgkmcnt(lgkm) (15 = do not wait), expcnt left alone
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (lgkm << 8); }
+
+// WM = waves along m: 4 (256 x 256 tile, eight waves) or 2 (256 (n) x 128 (m) tile, four waves, for problems with
+// so few 256 x 256 tiles that half the compute units would idle; same wave tile, same K order, same bits).
+template <bool RESID, bool QK, int WM = 4>
+__global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
+  constexpr int PW = 16 / WM;  // 1 KiB pieces of a W unit (256 rows) per wave; an A unit (64 WM rows) gives 4
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // Both problems' arguments are fetched together with the tile counts, in one round of scalar loads, and the
   // selected set is pinned in front of the early exit: left alone, the compiler sinks the argument loads below
@@ -372,19 +381,24 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;            // 0..7
-  const int wn = wave >> 2, wm = wave & 3;
+  const int wave = tid >> 6;            // 0..2 WM - 1
+  const int wn = wave / WM, wm = wave % WM;
   const int g = lane >> 5, li = lane & 31;
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * (64 * WM), n0 = tn * BN;
 
-  // async loads: per unit a wave issues 4 instructions for its 32 rows
+  // async loads: per unit a wave issues one instruction per 8 rows of its share
   const int ld_r = lane >> 3, ld_p = lane & 7;
-  uint32_t w_off[4], a_off[4];
+  uint32_t w_off[PW], a_off[4];
+#pragma unroll
+  for (int i = 0; i < PW; ++i) {
+    const int row = (wave * PW + i) * 8 + ld_r;
+    const int c = ld_p ^ ((row >> 1) & 7);
+    w_off[i] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.ldw + c * 16;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = (wave * 4 + i) * 8 + ld_r;
     const int c = ld_p ^ ((row >> 1) & 7);
-    w_off[i] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.ldw + c * 16;
     a_off[i] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.lda + c * 16;
   }
   const uint8_t* w_base = p.w + (int64_t)n0 * p.ldw;
@@ -401,7 +415,7 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   auto issue_load = [&](int j, int op, int i) {
     const int slot = (2 * j + op) % NSLOT;
     j = min(j, nu - 1);
-    const uint32_t dst = lds0 + slot * kUnitBytes + (wave_u * 4 + i) * 1024;
+    const uint32_t dst = lds0 + slot * kUnitBytes + (wave_u * (op ? 4 : PW) + i) * 1024;
     const uint8_t* ub = (op ? a_base : w_base) + (int64_t)j * UK;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
@@ -481,16 +495,17 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
   };
 
   // One step = 8 MFMAs per wave; the fragments of step 2j + par sit in fw and fa[par].  Between the MFMAs the
-  // wave reads the 12 fragments of the next step and issues 4 async loads of unit j + 2.  `loads` = false for
+  // wave reads the 12 fragments of the next step and issues its async loads of unit j + 2 (the even step the
+  // PW pieces of W, the odd step the 4 of A).  `loads` = false for
   // the last two units (nothing is left to fetch; the odd step then waits for everything in flight);
   // `last` = true for the very last step: no next fragments, and the registers they would occupy take the
   // epilogue's operands instead, whose latency the remaining MFMAs cover.
   auto step = [&](int j, int par, bool loads, bool last) {
     if (par) {
       if (loads)
-        __builtin_amdgcn_s_waitcnt(0x0074);  // vmcnt(4) lgkmcnt(0)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PW, 0));  // all but the W pieces the even step just issued; lgkmcnt(0)
       else
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));   // vmcnt(0) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
     } else {
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
@@ -505,8 +520,9 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
         read_w(j + par, par ^ 1, idx >> 1, 1);
       } else {
         read_a(par ^ 1, j + par, par ^ 1, idx >> 2, (idx >> 1) & 1);
-        if (loads) issue_load(j + 2, par, idx >> 1);
+        if (loads && (par || PW == 4)) issue_load(j + 2, par, idx >> 1);
       }
+      if (PW == 8 && !par && loads && !last) issue_load(j + 2, 0, idx);  // eight W pieces: one per slot
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -514,8 +530,8 @@ __global__ __launch_bounds__(512) void fp8_gemm_kernel(GemmPair q) {
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) issue_load(u >> 1, u & 1, i);
-  __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): W and A unit 0 have landed
+    for (int i = 0; i < ((u & 1) ? 4 : PW); ++i) issue_load(u >> 1, u & 1, i);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(PW + 4, 15));  // all but W and A unit 1: W and A unit 0 have landed
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
@@ -711,6 +727,12 @@ static int gemm_set_attributes() {
                             kMainLdsBytes) != hipSuccess ||
         hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             kMainLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, false, 2>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_kernel<true, false, 2>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, true, 2>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess ||
         hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
                             hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
       return (int)DSX_ELAUNCH;
@@ -730,6 +752,8 @@ static bool gemm_main_kernel_ok(dsx::GemmArgs& p) {
   return p.M > 8 && !p.w_row_scale && (p.K % 128) == 0 && vec_ok;
 }
 
+constexpr int kHalfTileThreshold = 128;
+
 // One launch of the main kernel over one or two problems (of the same kind: plain, residual or qk epilogue).
 static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStream_t st) {
   using namespace dsx;
@@ -738,6 +762,22 @@ static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStre
   q.p[1] = p1 ? *p1 : p0;
   q.total0 = p0.tiles_m * p0.tiles_n;
   q.total = q.total0 + (p1 ? p1->tiles_m * p1->tiles_n : 0);
+  // At most half the compute units' worth of 256 x 256 tiles (MI355X: 256): tiles of 128 token rows fill twice
+  // as many, and the four-wave form of the kernel runs them (same wave tile and K order: same bits).
+  if (q.total <= kHalfTileThreshold) {
+    q.p[0].tiles_m = (p0.M + 127) / 128;
+    q.p[1].tiles_m = p1 ? (p1->M + 127) / 128 : q.p[0].tiles_m;
+    q.total0 = q.p[0].tiles_m * p0.tiles_n;
+    q.total = q.total0 + (p1 ? q.p[1].tiles_m * p1->tiles_n : 0);
+    const int grid = ((q.total + 7) / 8) * 8;
+    if (p0.resid)
+      fp8_gemm_kernel<true, false, 2><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+    else if (p0.qk_heads > 0)
+      fp8_gemm_kernel<false, true, 2><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+    else
+      fp8_gemm_kernel<false, false, 2><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+    return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
+  }
   const int grid = ((q.total + 7) / 8) * 8;
   if (p0.resid)
     fp8_gemm_kernel<true, false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);

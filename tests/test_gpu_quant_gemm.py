@@ -294,3 +294,43 @@ def test_qk_epilogue_on_a_grouped_text_and_image_pair(dev):
                           qk=dict(heads=heads, q_norm_w=wq, k_norm_w=wk, rope=rope, pos0=pos0)))
     outs = ops.fp8_gemm_grouped(probs)
     assert torch.equal(outs[0], wants[0]) and torch.equal(outs[1], wants[1])
+
+
+@pytest.mark.parametrize("kind", ["plain", "residual", "qk"])
+def test_half_height_tiles_give_the_bits_of_full_tiles(dev, kind):
+    """A problem with at most 128 tiles of 256 x 256 runs on tiles of 128 token rows (four waves, twice as many
+    workgroups); one with more runs on 256-row tiles (eight waves).  Same wave tile and K order, so the rows of a
+    small problem equal the same rows inside a large one, bit for bit, for each of the three epilogues."""
+    from diffsynth_engine_amd import ops
+
+    K, N, M_big, M_small = 1024, 3072, 3000, 1000   # 12 x 12 = 144 tiles against 4 x 12 = 48 (-> 8 x 12 of 128 rows)
+    heads = 8
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(M_big, K, generator=g).bfloat16().to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(dev)
+    bias = torch.randn(N, generator=g).bfloat16().to(dev)
+    w8, ws = ops.quantize_weight_fp8(w)
+    xq, xs = ops.quantize_fp8(x)
+    kw_big, kw_small = {}, {}
+    if kind == "residual":
+        resid = torch.randn(M_big, N, generator=g).bfloat16().to(dev)
+        gate = torch.randn(1, N, generator=g).bfloat16().to(dev)
+        kw_big = dict(resid=resid, gate=gate, rows_per_batch=M_big)
+        kw_small = dict(resid=resid[:M_small], gate=gate, rows_per_batch=M_small)
+    elif kind == "qk":
+        ang = torch.rand(1, M_big, 64, generator=g) * 6.28
+        rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).float().to(dev)
+        nq, nk = [(1 + 0.2 * torch.randn(128, generator=g)).bfloat16().to(dev) for _ in range(2)]
+        qk = dict(heads=heads, q_norm_w=nq, k_norm_w=nk, rope=rope, pos0=0, eps=1e-6)
+        kw_big, kw_small = dict(rows_per_batch=M_big, qk=qk), dict(rows_per_batch=M_small, qk=qk)
+    big = ops.fp8_gemm(xq, w8, xs, ws, bias, **kw_big)
+    small = ops.fp8_gemm(xq[:M_small], w8, xs[:M_small], ws, bias, **kw_small)
+    assert torch.equal(small, big[:M_small])
+    # ragged heights around the 128-row tile, and a single partly filled tile
+    for m in (129, 127, 9):
+        kws = dict(kw_small)
+        if kind == "residual":
+            kws = dict(resid=kw_big["resid"][:m], gate=kw_big["gate"], rows_per_batch=m)
+        elif kind == "qk":
+            kws = dict(rows_per_batch=m, qk=kw_big["qk"])
+        assert torch.equal(ops.fp8_gemm(xq[:m], w8, xs[:m], ws, bias, **kws), big[:m]), m
