@@ -24,6 +24,8 @@
 //
 // LDS swizzles: K rows (256 B): 16-byte chunk c of key r at c ^ (r & 15)  (ds_read_b128 by 32 rows);
 //               V rows (256 B): chunk c of key r at c ^ ((r & 3) << 2)    (transposing 8-byte reads).
+#include <algorithm>
+
 #include "attn_internal.h"
 #include "common.h"
 
@@ -544,6 +546,9 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
 
 // Combines the parts of every split unit: O = sum_i O_i 2^(m_i - m), l likewise, m = max_i m_i.
 // Same lane <-> (query, d) mapping as the attention kernel, so the slots are read as they were written.
+// blockIdx.y picks one of the sixteen (dt, rq) groups of four output columns: a unit's merge is spread over
+// sixteen workgroups, each reading one 16-byte vector per lane and part (a unit cut into many parts would
+// otherwise be read, 128 KiB per part, by a single workgroup).
 __global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, AttnSplit sp) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 5, li = lane & 31;
@@ -551,6 +556,7 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, Attn
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int nkb = (int)((p.skv[0] + p.skv[1] + KB - 1) / KB);
   const int t = blockIdx.x;
+  const int dt = (int)blockIdx.y >> 2, rq = (int)blockIdx.y & 3;
   const int first_piece = (t * nkb) / sp.len, last_piece = ((t + 1) * nkb - 1) / sp.len;
   const int np = last_piece - first_piece + 1;
   if (np == 1) return;  // the unit was covered by one piece, which wrote the output itself
@@ -561,27 +567,26 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, Attn
   const int qi = wave * 32 + li;
   float m = -INFINITY;
   for (int i = 0; i < np; ++i) m = fmaxf(m, base[(int64_t)i * kSlotFloats + kSlotOFloats + QB + qi]);
-  f32x16 oacc[4];
-#pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  f32x4 o = {0.f, 0.f, 0.f, 0.f};
   float l = 0.f;
   for (int i = 0; i < np; ++i) {
     const float* slot = base + (int64_t)i * kSlotFloats;
     const float w = __builtin_amdgcn_exp2f(slot[kSlotOFloats + QB + qi] - m);
     l += slot[kSlotOFloats + qi] * w;
+    const f32x4 v = *reinterpret_cast<const f32x4*>(slot + ((((dt * 4 + rq) * 8 + wave) * 2 + g) * 32 + li) * 4);
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(slot + ((((dt * 4 + rq) * 8 + wave) * 2 + g) * 32 + li) * 4);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) oacc[dt][4 * rq + c] += v[c] * w;
-      }
+    for (int c = 0; c < 4; ++c) o[c] += v[c] * w;
   }
   const int64_t row = (int64_t)qblk * QB + qi;
-  if (row < Sq) store_output(p, b, h, row, g, oacc, 1.0f / l);
+  if (row >= Sq) return;
+  const float inv = 1.0f / l;
+  const int seg = row >= p.sq[0] ? 1 : 0;
+  uint16_t* dst = (uint16_t*)p.o[seg] + (int64_t)b * p.o_sb[seg] + (int64_t)h * p.o_sh[seg] +
+                  (row - (seg ? p.sq[0] : 0)) * p.o_ss[seg];
+  u32x2 w2;
+  w2.x = pack_bf16x2(o[0] * inv, o[1] * inv);
+  w2.y = pack_bf16x2(o[2] * inv, o[3] * inv);
+  *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w2;
 }
 
 }  // namespace
@@ -603,10 +608,20 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   // compute units runs at a higher clock (measured at 432 units on 256 compute units: 252 us whole,
   // 265 us split; at 384 units: 218 us whole, 207 us split).
   if (tail == 0 || nkb < 32 || (int64_t)(cus - tail) * 4 < rounds * cus) return 0;
+  // One piece per compute unit, but no more than eight per unit: every piece leaves 130 KiB of partial results
+  // that the merge reads back, and a handful of units cut into 256 slivers costs more there than it saves here.
+  const int pieces = (int)std::min<int64_t>(cus, (int64_t)tail * 8);
+  const int len = (int)(((int64_t)tail * nkb + pieces - 1) / pieces);
+  // What the split saves against what it costs, from measurements on this chip: a 64-key block of a workgroup
+  // takes ~1.65 us; a part (a piece, or the piece's share of a second unit) costs ~0.09 us of writing and reading
+  // back its 130 KiB, the merge launch ~8 us.  (2048 x 2048 x 24 heads = 192 units: 59 us whole, 85 us cut into
+  // 256 pieces of 24 blocks; 2816 x 2816 = 264 units: 144 us whole, 114 us with its last 8 units cut into 64.)
+  const double saved_us = (nkb - len) * 1.65, cost_us = (pieces + tail) * 0.09 + 8.0;
+  if (saved_us < 1.25 * cost_us) return 0;
   sp.full_units = (int)(units - tail);
   sp.tail_units = tail;
-  sp.pieces = cus;
-  sp.len = (int)(((int64_t)tail * nkb + cus - 1) / cus);
+  sp.pieces = pieces;
+  sp.len = len;
   sp.max_parts = (nkb + sp.len - 1) / sp.len + 1;
   return (int64_t)tail * sp.max_parts * kSlotFloats * (int64_t)sizeof(float);
 }
@@ -685,7 +700,7 @@ int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_b
     attn_plain_kernel<true, false, false><<<grid, block, kLdsBytes, st>>>(p, sp);
   if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
   if (sp.tail_units > 0) {
-    attn_merge_kernel<<<dim3((unsigned)sp.tail_units), block, 0, st>>>(p, sp);
+    attn_merge_kernel<<<dim3((unsigned)sp.tail_units, 16), block, 0, st>>>(p, sp);
     if (hipGetLastError() != hipSuccess) return DSX_ELAUNCH;
   }
   return DSX_OK;
