@@ -32,11 +32,13 @@ SCALE_SUFFIX = ".weight_scale"  # per-tensor scale of an already quantised weigh
 
 
 def _lora_factors(down: torch.Tensor, up: torch.Tensor, coef: float, n: int, k: int, dev):
-    """(down e4m3 (r', K), its scale, up e4m3 (N, r'), its scale x coef) with the rank zero-padded to r' % 16 == 0."""
+    """(down e4m3 (r', K), its scale, up e4m3 (N, r'), its scale x coef) with the rank zero-padded to a multiple of
+    128: the up product then has a whole 128-byte K unit and runs on the tile kernel with the residual epilogue
+    (13.8 us for 4608 x 3072 at rank 16) instead of the ragged-K kernel (45.8 us)."""
     if tuple(down.shape[1:]) != (k,) or up.shape[0] != n or up.shape[1] != down.shape[0]:
         raise ValueError("LoRA factors (%s, %s) do not fit a Linear %d -> %d" % (tuple(down.shape), tuple(up.shape), k, n))
     r = down.shape[0]
-    rp = (r + 15) // 16 * 16
+    rp = (r + 127) // 128 * 128  # a whole 128-byte K unit: both products then run on the tile kernel
     d = torch.zeros((rp, k), dtype=torch.bfloat16, device=dev)
     d[:r] = down.to(dev, torch.bfloat16)
     u = torch.zeros((n, rp), dtype=torch.bfloat16, device=dev)
@@ -64,8 +66,8 @@ class _Linear:
 
     def add_lora(self, down: torch.Tensor, up: torch.Tensor, coef: float):
         """Unfused low-rank update y += coef * up(down(x)) (models/basic/lora.py:29-32,137-141); both factors are
-        stored as e4m3 like every other Linear under fp8 inference.  The rank is zero-padded to a multiple of 16
-        (the GEMM's K granularity) and the coefficient is folded into the up factor's scale."""
+        stored as e4m3 like every other Linear under fp8 inference.  The rank is zero-padded (see _lora_factors)
+        and the coefficient is folded into the up factor's scale."""
         self.loras.append(_lora_factors(down, up, coef, self.n, self.k, self.w.device))
 
     def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None, qk=None):
@@ -78,15 +80,21 @@ class _Linear:
             return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch, qk))
         if qk is not None:  # the low-rank terms are added after the main product: q/k can only be prepared after them
             raise ValueError("a LoRA on a qkv projection needs qk_prep='attention'")
+        if resid is None:  # y = main + sum(lora): the low-rank products are added by residual epilogues
+            # the main product and the first down projection read the same operand and have the same (plain)
+            # epilogue: one launch, in which the few tiles of the projection run beside the main product's
+            dq, ds, _, _ = self.loras[0]
+            y, h0 = ops.fp8_gemm_grouped([self.problem(a_q, a_s, out),
+                                          dict(a_q=a_q, w_q=dq, a_scale=a_s, w_scale=ds, bias=None)])
+            hs_list = [h0] + [ops.fp8_gemm(a_q, dq, a_s, ds, None) for dq, ds, _, _ in self.loras[1:]]
+            for h, (_, _, uq, us) in zip(hs_list, self.loras):
+                hq, hs = ops.quantize_fp8(h, scaled=True)
+                ops.fp8_gemm(hq, uq, hs, us, None, resid=y, out=y)
+            return y
         lows = []
         for dq, ds, uq, us in self.loras:
             hq, hs = ops.quantize_fp8(ops.fp8_gemm(a_q, dq, a_s, ds, None), scaled=True)
             lows.append((hq, hs, uq, us))
-        if resid is None:  # y = main + sum(lora): the low-rank products are added by residual epilogues
-            y = ops.fp8_gemm(**self.problem(a_q, a_s, out))
-            for hq, hs, uq, us in lows:
-                ops.fp8_gemm(hq, uq, hs, us, None, resid=y, out=y)
-            return y
         # resid + gate*(main + lora) = (resid + gate*lora) + gate*main: every term rides a GEMM epilogue
         acc = resid
         for hq, hs, uq, us in lows:
