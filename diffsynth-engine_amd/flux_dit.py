@@ -301,14 +301,10 @@ class FluxDiTRunner:
 
     def _modulate_q(self, x, scale, shift):
         """LayerNorm-modulate straight to the GEMM operand format."""
-        if self.scaled:
-            return ops.adaln_modulate(x, scale, shift, EPS, want_bf16=False, want_fp8=True)
-        return ops.quantize_fp8(ops.adaln_modulate(x, scale, shift, EPS), scaled=False)
+        return ops.adaln_modulate(x, scale, shift, EPS, want_bf16=False, want_fp8=True, scaled=self.scaled)
 
     def _gelu_q(self, h):
-        if self.scaled:
-            return ops.gelu_tanh(h, want_bf16=False, want_fp8=True)
-        return ops.quantize_fp8(ops.gelu_tanh(h), scaled=False)
+        return ops.gelu_tanh(h, want_bf16=False, want_fp8=True, scaled=self.scaled)
 
     # ------------------------------------------------------------------ blocks
     def _joint_block(self, i: int, img, txt, mod_a, mod_b, rope):
@@ -411,11 +407,7 @@ class FluxDiTRunner:
                                eps=EPS, out=att.transpose(1, 2), score_bound=self.score_bound.get(pre, 0.0))
         # cat([attention, gelu(mlp)]) (flux_dit.py:315-317) is never materialised in bf16: one kernel reads both
         # parts and emits the e4m3 operand of proj_out with its per-token scale
-        if self.scaled:
-            q, sc = ops.concat_gelu_tanh(att.view(B * S, d), h[:, 3 * d:], want_fp8=True)
-        else:
-            q, sc = ops.quantize_fp8(ops.concat_gelu_tanh(att.view(B * S, d), h[:, 3 * d:], want_bf16=True,
-                                                          want_fp8=False), scaled=False)
+        q, sc = ops.concat_gelu_tanh(att.view(B * S, d), h[:, 3 * d:], want_fp8=True, scaled=self.scaled)
         out = L[pre + "proj_out"](q, sc, resid=x.reshape(B * S, d), gate=gate, rows_per_batch=S)
         return out.view(B, S, d)
 

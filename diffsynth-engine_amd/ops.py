@@ -448,10 +448,11 @@ def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, rope:
 
 def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Optional[torch.Tensor],
                    eps: float = 1e-6, ln_weight=None, ln_bias=None, want_bf16: bool = True,
-                   want_fp8: bool = False):
+                   want_fp8: bool = False, scaled: bool = True):
     """LayerNorm(x) * (1 + scale) + shift per token; x (B,S,D) bf16, scale/shift (B,D) or (B,1,D) bf16.
 
-    Returns y (bf16) and/or (q e4m3, q_scale fp32 per token) depending on want_*.
+    Returns y (bf16) and/or (q e4m3, q_scale fp32 per token) depending on want_*; ``scaled=False``: q is the
+    reference's bare cast of y (unit scale, utils/fp8_linear.py:35) and q_scale is None.
     """
     _require_cuda(x)
     if x.dtype != _BF16:
@@ -488,7 +489,7 @@ def adaln_modulate(x: torch.Tensor, scale: Optional[torch.Tensor], shift: Option
     _require_cuda(scale_t, shift_t, ln_weight, ln_bias)
     y = torch.empty((rows, D), dtype=_BF16, device=x.device) if want_bf16 else None
     q = torch.empty((rows, D), dtype=FP8, device=x.device) if want_fp8 else None
-    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
+    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 and scaled else None
     rc = _lib.load().dsx_adaln_modulate(_ptr(x2), ldx, _ptr(scale_t), _ptr(shift_t), mod_sb, max(rows // B, 1),
                                         _ptr(ln_weight), _ptr(ln_bias), eps, _ptr(y), D, _ptr(q), D, _ptr(qs), rows,
                                         D, _stream())
@@ -535,9 +536,9 @@ def gated_residual(x: torch.Tensor, y: torch.Tensor, gate: Optional[torch.Tensor
 
 
 def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, out: Optional[torch.Tensor] = None,
-              erf: bool = False):
+              erf: bool = False, scaled: bool = True):
     """tanh-GELU (``erf``: the exact erf form of nn.GELU()) over the last dim of a bf16 tensor (a column slice of
-    a wider buffer is fine)."""
+    a wider buffer is fine).  ``scaled=False``: the e4m3 output is the bare cast (unit scale, q_scale None)."""
     _require_cuda(x, out)
     if x.dtype != _BF16:
         raise ValueError("gelu_tanh expects bf16")
@@ -552,7 +553,7 @@ def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, o
         else:
             y = torch.empty((rows, D), dtype=_BF16, device=x.device)
     q = torch.empty((rows, D), dtype=FP8, device=x.device) if want_fp8 else None
-    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
+    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 and scaled else None
     fn = _lib.load().dsx_gelu_erf if erf else _lib.load().dsx_gelu_tanh
     _lib.check(fn(_ptr(x2), ldx, _ptr(y), ldy, _ptr(q), D, _ptr(qs), rows, D, _stream()),
                "dsx_gelu_erf" if erf else "dsx_gelu_tanh")
@@ -564,8 +565,10 @@ def gelu_tanh(x: torch.Tensor, want_bf16: bool = True, want_fp8: bool = False, o
     return res[0] if len(res) == 1 else tuple(res)
 
 
-def concat_gelu_tanh(prefix: torch.Tensor, x: torch.Tensor, want_bf16: bool = False, want_fp8: bool = True):
-    """[prefix | gelu_tanh(x)] along the last dim for 2-D (rows, D) views; bf16 and/or per-token e4m3 output."""
+def concat_gelu_tanh(prefix: torch.Tensor, x: torch.Tensor, want_bf16: bool = False, want_fp8: bool = True,
+                     scaled: bool = True):
+    """[prefix | gelu_tanh(x)] along the last dim for 2-D (rows, D) views; bf16 and/or per-token e4m3 output
+    (``scaled=False``: the bare cast, q_scale None)."""
     _require_cuda(prefix, x)
     if prefix.dtype != _BF16 or x.dtype != _BF16 or prefix.dim() != 2 or x.dim() != 2:
         raise ValueError("concat_gelu_tanh expects 2-D bf16 tensors")
@@ -576,7 +579,7 @@ def concat_gelu_tanh(prefix: torch.Tensor, x: torch.Tensor, want_bf16: bool = Fa
     Dt = Dp + D
     y = torch.empty((rows, Dt), dtype=_BF16, device=x.device) if want_bf16 else None
     q = torch.empty((rows, Dt), dtype=FP8, device=x.device) if want_fp8 else None
-    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 else None
+    qs = torch.empty((rows,), dtype=torch.float32, device=x.device) if want_fp8 and scaled else None
     rc = _lib.load().dsx_concat_gelu_tanh(_ptr(p2), ldp, Dp, _ptr(x2), ldx, _ptr(y), Dt, _ptr(q), Dt, _ptr(qs), rows,
                                           D, _stream())
     _lib.check(rc, "dsx_concat_gelu_tanh")

@@ -86,11 +86,8 @@ class WanDiTRunner:
         return ops.quantize_fp8(y, scaled=self.scaled)
 
     def _modulate_q(self, x, scale, shift, w=None, b=None):
-        if self.scaled:
-            return ops.adaln_modulate(x, scale, shift, self.cfg["eps"], ln_weight=w, ln_bias=b, want_bf16=False,
-                                      want_fp8=True)
-        return ops.quantize_fp8(ops.adaln_modulate(x, scale, shift, self.cfg["eps"], ln_weight=w, ln_bias=b),
-                                scaled=False)
+        return ops.adaln_modulate(x, scale, shift, self.cfg["eps"], ln_weight=w, ln_bias=b, want_bf16=False,
+                                  want_fp8=True, scaled=self.scaled)
 
     def rope_table(self, f, h, w, theta=10000.0):
         """(1, f*h*w, 64, 2) fp32 (cos, sin): head dim split (d - 2*(d//3), d//3, d//3) over (frame, row, col)
@@ -175,10 +172,7 @@ class WanDiTRunner:
         # feed-forward
         hq, hs = self._modulate_q(x2.view(B, S, d), m[4], m[3])
         h = L[p + "ffn.0"](hq.view(B * S, d), hs)
-        if self.scaled:
-            gq, gs = ops.gelu_tanh(h, want_bf16=False, want_fp8=True)
-        else:
-            gq, gs = ops.quantize_fp8(ops.gelu_tanh(h), scaled=False)
+        gq, gs = ops.gelu_tanh(h, want_bf16=False, want_fp8=True, scaled=self.scaled)
         x2 = L[p + "ffn.2"](gq, gs, resid=x2, gate=m[5], rows_per_batch=S)
         return x2.view(B, S, d)
 

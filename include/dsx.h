@@ -294,7 +294,9 @@ int dsx_rmsnorm_rows(const void* x, int64_t ldx, const void* w, float eps, const
  * models/wan/wan_dit.py:25-26,188,191,236.
  *   x: (B*S, D) bf16 (ldx); scale, shift: bf16 (D,) per batch entry, batch stride mod_sb
  *   (row r uses batch r / rows_per_batch); ln_w/ln_b: optional bf16 affine (Wan norm3) or NULL.
- *   y_bf16 (ldy) and/or (q_fp8 (ldq) + q_scale[rows]) are written; either may be NULL.
+ *   y_bf16 (ldy) and/or (q_fp8 (ldq) + q_scale[rows]) are written; either may be NULL.  q without q_scale is the
+ *   reference's bare cast (utils/fp8_linear.py:35): unit scale, values beyond e4m3's range become NaN (this holds
+ *   for dsx_gelu_tanh, dsx_gelu_erf and dsx_concat_gelu_tanh too).
  *   Rounding follows the bf16 op sequence: bf16(LN) -> bf16(1+scale) -> bf16(mul) -> bf16(add).
  *   D % 8 == 0, D <= 16384.
  */

@@ -199,3 +199,32 @@ def test_empty_inputs_are_accepted(dev):
     assert ops.gelu_tanh(x).shape == (0, 3072)
     mod = torch.zeros(1, 3072, dtype=torch.bfloat16, device=dev)
     assert ops.adaln_modulate(x.view(1, 0, 3072), mod, mod, 1e-6).shape == (1, 0, 3072)
+
+
+def test_fused_kernels_emit_the_bare_cast_without_a_scale(dev):
+    """``scaled=False`` (no q_scale): the e4m3 output of AdaLN-modulate, GELU and concat-GELU is the reference's bare
+    cast of their bf16 output (utils/fp8_linear.py:35), bit for bit what the stand-alone cast kernel gives, NaN
+    codes beyond the format's range included."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(21)
+    for rows, D in ((300, 3072), (77, 1024), (40, 5120)):
+        x = (torch.randn(1, rows, D, generator=g) * 3).bfloat16().to(dev)
+        x[0, 0, :8] = torch.tensor([600.0, -600.0, 470.0, 460.0, 448.0, 1e-3, -0.0, 2e-3]).bfloat16()  # around the edges
+        scale = (torch.randn(1, D, generator=g) * 2).bfloat16().to(dev)
+        shift = (torch.randn(1, D, generator=g) * 50).bfloat16().to(dev)
+        y = ops.adaln_modulate(x, scale, shift, 1e-6)
+        q, qs = ops.adaln_modulate(x, scale, shift, 1e-6, want_bf16=False, want_fp8=True, scaled=False)
+        want, _ = ops.quantize_fp8(y.view(rows, D), scaled=False)
+        assert qs is None and torch.equal(q.view(rows, D).view(torch.uint8), want.view(torch.uint8))
+        big = (x.view(rows, D).float() * 200).bfloat16()   # GELU keeps large positive values: some exceed 448
+        yg = ops.gelu_tanh(big)
+        qg, qsg = ops.gelu_tanh(big, want_bf16=False, want_fp8=True, scaled=False)
+        wantg, _ = ops.quantize_fp8(yg, scaled=False)
+        assert qsg is None and torch.equal(qg.view(torch.uint8), wantg.view(torch.uint8))
+        assert (wantg.view(torch.uint8) & 0x7F == 0x7F).any()  # the NaN code occurs in this set-up
+        pre = (torch.randn(rows, 256, generator=g) * 100).bfloat16().to(dev)
+        yc = ops.concat_gelu_tanh(pre, big, want_bf16=True, want_fp8=False)
+        qc, qsc = ops.concat_gelu_tanh(pre, big, want_fp8=True, scaled=False)
+        wantc, _ = ops.quantize_fp8(yc, scaled=False)
+        assert qsc is None and torch.equal(qc.view(torch.uint8), wantc.view(torch.uint8))
