@@ -695,6 +695,25 @@ def main():
     if not args.no_micro:
         result["detail"].update(micro_benchmarks(torch, ops, dev))
         result["detail"]["mfma_ceiling_probe"] = mfma_ceiling(torch, dev)
+        # the same model at other image sizes (512 text tokens): two warm-up steps, three timed ones each
+        other = {}
+        for side in (64, 96, 192):
+            inp_o = dict(inp, hidden_states=torch.randn(1, 16, side, side, generator=g, device=dev).to(torch.bfloat16))
+            for _ in range(2):
+                runner(**inp_o)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                out_o = runner(**inp_o)
+            torch.cuda.synchronize()
+            ms_o = (time.perf_counter() - t0) * 1e3 / 3
+            assert torch.isfinite(out_o.float()).all().item(), "non-finite output"
+            tokens = side * side // 4 + N_TXT
+            gemm_o, attn_o = step_flops(args.double, args.single, n_img=side * side // 4)
+            ideal_o = gemm_o / PEAK_FP8 + attn_o / PEAK_BF16
+            other["%dx%d" % (side * 8, side * 8)] = {
+                "tokens": tokens, "ms_per_step": round(ms_o, 2), "step_roofline_frac": round(ideal_o * 1e3 / ms_o, 4)}
+        result["detail"]["flux_other_image_sizes"] = other
     del runner
     torch.cuda.empty_cache()
     if not args.no_micro:
