@@ -33,14 +33,17 @@ N_IMG, N_TXT = 4096, 512
 
 def flux_state_dict_stream(num_double, num_single, device, seed=0, std=0.02):
     """Yield (name, tensor) pairs of a random Flux.1-dev-architecture DiT, generated on the device one tensor
-    at a time (weights N(0,std) bf16, biases 0, RMSNorm weights 1) so that the runner can quantise as it goes."""
+    at a time (weights N(0,std) bf16, biases 0, RMSNorm weights 1) so that the runner can quantise as it goes.
+    std=None draws every Linear N(0, 1/fan_in) instead (AdaLN projections at half that deviation): every layer's
+    output then stays O(1), far below e4m3's 448, which the reference's unscaled casts need."""
     import torch
 
     g = torch.Generator(device=device).manual_seed(seed)
     d = HIDDEN
 
     def lin(name, n_in, n_out):
-        yield name + ".weight", (torch.randn(n_out, n_in, generator=g, device=device) * std).to(torch.bfloat16)
+        s = std if std is not None else (0.5 if "norm" in name else 1.0) / n_in ** 0.5
+        yield name + ".weight", (torch.randn(n_out, n_in, generator=g, device=device) * s).to(torch.bfloat16)
         yield name + ".bias", torch.zeros(n_out, dtype=torch.bfloat16, device=device)
 
     def ones(name):

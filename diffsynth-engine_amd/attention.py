@@ -20,6 +20,9 @@ SUPPORTED_IMPLEMENTATIONS = ("sdpa", "mi355x")
 
 
 def _prep(t: torch.Tensor) -> torch.Tensor:
+    """The kernel computes on bf16 operands (fp32 accumulation and softmax).  fp32 / fp16 tensors are rounded to
+    bf16 once here, which is narrower than torch's SDPA would compute for them; the result stays within the bar the
+    bf16 path is held to (2e-2 of the row maximum against fp32 SDPA of the unrounded inputs, tested)."""
     if t.dtype != torch.bfloat16:
         t = t.to(torch.bfloat16)
     if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:

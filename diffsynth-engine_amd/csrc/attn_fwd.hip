@@ -195,7 +195,10 @@ extern "C" int64_t dsx_attn_workspace_bytes(const dsx_attn_params* p) {
   if (!p || p->head_dim != HD || p->batch <= 0 || p->heads <= 0) return 0;
   const int64_t Sq = p->sq[0] + p->sq[1], Skv = p->skv[0] + p->skv[1];
   if (Sq <= 0 || Skv <= 0 || Sq > (1ll << 30) || Skv > (1ll << 30)) return 0;
-  return attn_k_copy_bytes(p) + attn_plain_workspace_bytes(*p);
+  // A call that copies k launches the attention kernel without scratch of its own (attn_run), so the copy is all
+  // it needs; only a call without a copy can use scratch for the key-range split.
+  const int64_t copy_bytes = attn_k_copy_bytes(p);
+  return copy_bytes > 0 ? copy_bytes : attn_plain_workspace_bytes(*p);
 }
 
 // ---- the allocation-free twin: the same launches over a static device array ------------------------------

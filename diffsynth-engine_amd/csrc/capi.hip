@@ -86,7 +86,10 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
 extern "C" int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_t iters, int32_t workgroups,
                                       void* sink, int64_t* flops_out, void* stream) {
   if (!operand_bits || !sink) return DSX_ENULL;
-  if (kind < 0 || kind > 7 || iters <= 0 || iters > (1ll << 32) || workgroups <= 0 || workgroups > (1 << 20))
+  // Caps: 2^22 iterations of four dependent MFMAs on 2^14 workgroups are already seconds of work; anything larger
+  // would keep the device busy for minutes, which callers sharing it cannot tell from a hang.
+  if (kind < 0 || kind > 7 || iters <= 0 || iters > DSX_PROBE_MAX_ITERS || workgroups <= 0 ||
+      workgroups > DSX_PROBE_MAX_WORKGROUPS)
     return DSX_EBADSHAPE;
   if ((uintptr_t)operand_bits & 3) return DSX_EALIGN;
   const dim3 grid((unsigned)workgroups), block(256);

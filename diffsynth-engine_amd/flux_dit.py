@@ -426,6 +426,11 @@ class FluxDiTRunner:
             image_ids[..., 1] += torch.arange(Hh // 2, device=dev)[:, None]
             image_ids[..., 2] += torch.arange(Ww // 2, device=dev)[None, :]
             image_ids = image_ids.reshape(1, -1, 3).repeat(text_ids.shape[0], 1, 1)
+        for name, ids in (("text_ids", text_ids), ("image_ids", image_ids)):
+            if ids.shape[0] not in (1, B):
+                raise ValueError("%s has batch %d beside latents of batch %d" % (name, ids.shape[0], B))
+        if text_ids.shape[0] != image_ids.shape[0]:  # one of them broadcasts: the RoPE table is built per entry
+            text_ids, image_ids = (t.expand(B, *t.shape[1:]) for t in (text_ids, image_ids))
         cond = self._timestep_mlp("time_embedder", timestep)
         if self.has_guidance and guidance is not None:
             cond = cond + self._timestep_mlp("guidance_embedder", guidance * 1000)

@@ -153,6 +153,11 @@ def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, res
         if rope is not None:
             if rope.dtype != torch.float32 or rope.dim() != 4 or rope.shape[2:] != (64, 2):
                 raise ValueError("rope table must be fp32 (B|1, S, 64, 2)")
+            # the kernel takes table row (m / rows_per_batch) of the batch axis on trust: it must be there
+            batches = -(-M // prob.rows_per_batch)
+            if rope.shape[0] not in (1, batches):
+                raise ValueError("fp8_gemm: a rope table of batch %d beside %d batch entries of %d rows"
+                                 % (rope.shape[0], batches, prob.rows_per_batch))
             rope = rope.contiguous()
             prob.rope, prob.rope_rows = _ptr(rope), rope.shape[1]
             prob.rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0

@@ -356,7 +356,11 @@ int dsx_flow_match_euler_step(const void* latents, const void* v, float dt, void
  * operand_bits (16 x 256 dwords, device memory; all zero or random, which changes power draw and with it the clock),
  * with no memory traffic inside the loop.  *flops_out (host memory, may be NULL) receives the flops of the launch; the
  * caller times it.  sink: one device float (never written for finite inputs).
+ * iters <= DSX_PROBE_MAX_ITERS and workgroups <= DSX_PROBE_MAX_WORKGROUPS, DSX_EBADSHAPE beyond: one launch at the
+ * caps is seconds of device time, and a longer one cannot be told from a hang by whoever shares the device.
  */
+#define DSX_PROBE_MAX_ITERS (1ll << 22)
+#define DSX_PROBE_MAX_WORKGROUPS (1 << 14)
 int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_t iters, int32_t workgroups, void* sink,
                            int64_t* flops_out, void* stream);
 

@@ -39,7 +39,9 @@ def _both(dev, H, S, fused, seed):
     g = torch.Generator().manual_seed(seed)
     q, k, v = [torch.randn(1, H, S, 128, generator=g).bfloat16().to(dev) for _ in range(3)]
     rope = wq = wk = None
-    if fused:
+    if fused == "k_only":  # only k is normalised: a k copy, no q work, and a unit count that would take the key split
+        wk = (1 + 0.1 * torch.randn(128, generator=g)).bfloat16().to(dev)
+    elif fused:
         ids = torch.zeros(1, S, 3)
         ids[0, :, 1] = torch.arange(S) // 16
         ids[0, :, 2] = torch.arange(S) % 16
@@ -78,6 +80,23 @@ def test_static_scratch_entry_point_equals_the_workspace_one_on_two_calls_in_a_r
         assert torch.isfinite(o_static.float()).all().item()
         assert o_static.float().abs().max().item() > 0
         assert torch.equal(o_static, o_ws), (fused, H, S)
+
+
+def test_a_call_that_copies_k_asks_for_the_copy_only(dev):
+    """With a k copy the attention kernel runs without scratch of its own, so the copy is all the call needs: the
+    size query must not add the key-range split's bytes (which a plain call of this shape does ask for), and both
+    entry points agree on two calls in a row."""
+    from diffsynth_engine_amd import _lib
+
+    lib = _lib.load()
+    for i, (H, S) in enumerate([(3, 2048), (1, 2048)]):
+        z = torch.zeros(1, H, S, 128, dtype=torch.bfloat16, device=dev)
+        w = torch.ones(128, dtype=torch.bfloat16, device=dev)
+        assert lib.dsx_attn_workspace_bytes(_params(_lib, z, z, z, z)) > 0          # plain: the split's scratch
+        assert lib.dsx_attn_workspace_bytes(_params(_lib, z, z, z, z, wk=w)) == 2 * H * S * 128
+        o_static, o_ws = _both(dev, H, S, "k_only", seed=50 + i)
+        assert o_static.float().abs().max().item() > 0
+        assert torch.equal(o_static, o_ws), (H, S)
 
 
 def test_static_scratch_entry_point_refuses_what_does_not_fit(dev):
