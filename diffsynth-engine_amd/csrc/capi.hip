@@ -1,6 +1,8 @@
 // Library-level entry points: ABI version, error strings, device check.
 #include <string.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 extern "C" int dsx_abi_version(void) { return DSX_ABI_VERSION; }
@@ -30,55 +32,54 @@ extern "C" int dsx_check_device(void) {
 // What the chip sustains with nothing but matrix instructions in flight, for the operand bits the caller supplies
 // (all-zero operands run at the full clock; random bits draw more power and the clock management lowers the clock).
 namespace dsx {
+// KIND 0 / 1: v_mfma_f32_32x32x16_bf16 / v_mfma_scale_f32_32x32x64_f8f6f4 (sixteen accumulator registers each);
+// KIND 2 / 3: v_mfma_f32_16x16x32_bf16 / v_mfma_scale_f32_16x16x128_f8f6f4 (four accumulator registers each, eight
+// independent accumulators, so that a wavefront has the same number of MFMAs in flight between two uses of one).
 template <int KIND, bool ROT = false>
 __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __restrict__ bits, int64_t iters,
                                                            float* __restrict__ sink) {
-  // eight operand dwords per lane (bf16: 4 + 4 are used; fp8: 8 + 8), the same for every workgroup
+  // eight operand dwords per lane and operand (bf16: 4 + 4 are used; fp8: 8 + 8), the same for every workgroup
   uint32_t r[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) r[i] = bits[i * 256 + threadIdx.x];
-  f32x16 acc[4];
+  constexpr bool kSmall = KIND >= 2;
+  constexpr int kAcc = kSmall ? 8 : 4;
+  typedef typename std::conditional<kSmall, f32x4, f32x16>::type acc_t;
+  acc_t acc[kAcc];
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < kAcc; ++t)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[t][e] = 0.f;
+    for (int e = 0; e < (kSmall ? 4 : 16); ++e) acc[t][e] = 0.f;
   for (int64_t it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {  // four independent accumulators
-      constexpr int kA = 0;
-      const int ra = ROT ? t : kA;  // ROT: the first operand changes from one MFMA to the next as well
-      if (KIND == 0) {
-        const u32x4 a = {r[ra], r[ra + 1], r[ra + 2], r[ra + 3]}, b = {r[8 + t], r[9 + t], r[10 + t], r[11 + t]};
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
-                                                         acc[t], 0, 0, 0);
-      } else if (KIND == 1) {
-        const i32x8 a = {(int)r[ra], (int)r[ra + 1], (int)r[ra + 2], (int)r[ra + 3], (int)r[ra + 4], (int)r[ra + 5],
-                         (int)r[ra + 6], (int)r[ra + 7]};
-        const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
-                         (int)r[15 - (t >> 1)]};
-        acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
-      } else if (KIND == 2) {
-        // the 16x16 shapes: the same operand registers, a quarter of the accumulator (the first four floats)
-        const u32x4 a = {r[ra], r[ra + 1], r[ra + 2], r[ra + 3]}, b = {r[8 + t], r[9 + t], r[10 + t], r[11 + t]};
-        f32x4 c = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-        acc[t][0] = c[0]; acc[t][1] = c[1]; acc[t][2] = c[2]; acc[t][3] = c[3];
+    for (int t = 0; t < kAcc; ++t) {  // independent accumulators
+      const int ra = ROT ? (t & 3) : 0;  // ROT: the first operand changes from one MFMA to the next as well
+      const int tb = t & 3;
+      if constexpr (KIND == 0 || KIND == 2) {
+        const u32x4 a = {r[ra], r[ra + 1], r[ra + 2], r[ra + 3]}, b = {r[8 + tb], r[9 + tb], r[10 + tb], r[11 + tb]};
+        if constexpr (KIND == 0)
+          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                           acc[t], 0, 0, 0);
+        else
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                           acc[t], 0, 0, 0);
       } else {
         const i32x8 a = {(int)r[ra], (int)r[ra + 1], (int)r[ra + 2], (int)r[ra + 3], (int)r[ra + 4], (int)r[ra + 5],
                          (int)r[ra + 6], (int)r[ra + 7]};
-        const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (t & 1)], (int)r[13], (int)r[14],
-                         (int)r[15 - (t >> 1)]};
-        f32x4 c = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-        c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
-        acc[t][0] = c[0]; acc[t][1] = c[1]; acc[t][2] = c[2]; acc[t][3] = c[3];
+        const i32x8 b = {(int)r[8], (int)r[9], (int)r[10], (int)r[11], (int)r[12 + (tb & 1)], (int)r[13], (int)r[14],
+                         (int)r[15 - (tb >> 1)]};
+        if constexpr (KIND == 1)
+          acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
+        else
+          acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[t], 0, 0, 0, 0, 0, 0);
       }
     }
   }
   float s = 0.f;
 #pragma unroll
-  for (int t = 0; t < 4; ++t)
+  for (int t = 0; t < kAcc; ++t)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) s += acc[t][e];
+    for (int e = 0; e < (kSmall ? 4 : 16); ++e) s += acc[t][e];
   if (s == 12345.678f) sink[0] = s;  // keeps the loop alive; never true for the inputs of the probe
 }
 }  // namespace dsx
@@ -107,6 +108,7 @@ extern "C" int dsx_mfma_ceiling_probe(int kind, const void* operand_bits, int64_
   }
 #undef DSX_PROBE
   const int64_t flops_per_mfma[4] = {2ll * 32 * 32 * 16, 2ll * 32 * 32 * 64, 2ll * 16 * 16 * 32, 2ll * 16 * 16 * 128};
-  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * 4 * flops_per_mfma[kind & 3];
+  const int64_t mfmas_per_iter = (kind & 3) >= 2 ? 8 : 4;  // the small shapes run eight independent accumulators
+  if (flops_out) *flops_out = (int64_t)workgroups * 4 * iters * mfmas_per_iter * flops_per_mfma[kind & 3];
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }

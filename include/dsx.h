@@ -349,10 +349,11 @@ int dsx_flow_match_euler_step(const void* latents, const void* v, float dt, void
 
 /*
  * Diagnostic, no counterpart in the reference: the on-box microbenchmark behind the roofline denominators.
- * Launches `workgroups` workgroups of four wavefronts that each run `iters` x 4 MFMAs (kind 0:
- * v_mfma_f32_32x32x16_bf16, kind 1: v_mfma_f32_32x32x64 on e4m3 operands, kinds 2 and 3: the 16x16x32 bf16 and
- * 16x16x128 e4m3 shapes, same operand registers; kind + 4: the first operand changes from one MFMA to the next as
- * well, as it does in a real kernel) on register operands taken from
+ * Launches `workgroups` workgroups of four wavefronts that each run `iters` rounds of MFMAs on independent
+ * accumulators (kind 0: v_mfma_f32_32x32x16_bf16, kind 1: v_mfma_f32_32x32x64 on e4m3 operands, four per round;
+ * kinds 2 and 3: the 16x16x32 bf16 and 16x16x128 e4m3 shapes, same operand registers, eight per round; kind + 4:
+ * the first operand changes from one MFMA to the next as well, as it does in a real kernel) on register operands
+ * taken from
  * operand_bits (16 x 256 dwords, device memory; all zero or random, which changes power draw and with it the clock),
  * with no memory traffic inside the loop.  *flops_out (host memory, may be NULL) receives the flops of the launch; the
  * caller times it.  sink: one device float (never written for finite inputs).
