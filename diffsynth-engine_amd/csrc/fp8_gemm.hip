@@ -1,18 +1,21 @@
 // FP8 e4m3 scaled GEMM for gfx950:  out = bf16((A * W^T) * a_scale[m] * w_scale + bias[n]).
 //
-// Both operands are K-contiguous, which is what v_mfma_f32_32x32x64_f8f6f4 wants: lane
-// (g = lane/32, i = lane%32) feeds 32 K-bytes of row i of the first operand and of column i of
+// Both operands are K-contiguous, which is what v_mfma_f32_16x16x128_f8f6f4 wants: lane
+// (q = lane/16, i = lane%16) feeds 32 K-bytes of row i of the first operand and of column i of
 // the second.  Any permutation of K applied to both operands leaves the product unchanged, so
 // the loaders only have to keep the two consistent.
+// (On random e4m3 operands, where the chip runs at its power limit, a bare stream of this shape sustains 9 % more
+// than one of v_mfma_f32_32x32x64_f8f6f4 -- 4.13 against 3.79 PFLOP/s -- while both reach the 5.0 PFLOP/s peak on
+// all-zero operands; the generic kernel for odd shapes below still uses the larger shape.)
 //
 // The kernels compute C^T tiles (first operand = W rows, second = A rows): the accumulator of
-// lane (g, j) then holds ONE token m = j and four consecutive output features per register
-// quad, so the per-token scale is a per-lane constant and the bf16 results leave as 8-byte stores.
+// lane (q, i) then holds ONE token m = i and four consecutive output features, so the per-token
+// scale is a per-lane constant and the bf16 results leave as 8-byte pieces.
 //
-// Main kernel: 256x256 output tile per workgroup, 8 waves as 2x4, each wave 128x64 = 4x2 MFMA
+// Main kernel: 256x256 output tile per workgroup, 8 waves as 2x4, each wave 128 (n) x 64 (m) = 8x4 MFMA
 // tiles (128 fp32 accumulators), two waves per SIMD.  Operands reach LDS by global_load_lds_dwordx4
 // (HBM/L2 -> LDS without staging registers) in 128-byte-wide units through a five-slot ring; MFMA
-// operand fragments are read one step ahead so that LDS reads overlap the MFMAs.  LDS rows are
+// operand fragments are read ahead of their use so that LDS reads overlap the MFMAs.  LDS rows are
 // 128 B (8 chunks of 16 B); chunk c of row r lives at chunk c ^ ((r/2)&7), which makes 16 lanes
 // reading 16 consecutive rows at one logical chunk hit 16 distinct bank groups.
 // One launch can carry two independent problems (the image- and text-stream linears of a joint
@@ -191,44 +194,47 @@ __device__ __forceinline__ int unit_off(int row, int chunk) {
 // (256 rows x 128 B = 32 KiB), so that every async load instruction (64 lanes x 16 B) fetches
 // eight whole 128-byte cache lines: with 64-byte rows each line would be requested twice, a step
 // apart, and the second request stalls the L1 behind the still-pending first one.  Five unit
-// slots (160 KiB) form a ring W0 A0 W1 A1 W2 | A2 W3 ...; one MFMA step consumes 64 bytes of K,
-// i.e. half of a W unit and half of an A unit.
-// Eight waves as 2 (n) x 4 (m), each 128 (n) x 64 (m) = 4x2 MFMA tiles (128 accumulators), so that two
-// waves share a SIMD: while one waits at the step's barrier or for its operands, the other's MFMAs keep
-// the matrix pipe busy, and the two overlap their epilogues.  (Four waves of 128 x 128 read a third
-// fewer fragment bytes per MFMA but leave the pipe idle in those waits: 3-12 % slower.)
+// slots (160 KiB) form a ring W0 A0 W1 A1 W2 | A2 W3 ...; one unit is one K extent of the MFMA.
+// Eight waves as 2 (n) x 4 (m), each 128 (n) x 64 (m) = 8x4 MFMA tiles (128 accumulators), so that two
+// waves share a SIMD: while one waits at the unit's barrier or for its operands, the other's MFMAs keep
+// the matrix pipe busy, and the two overlap their epilogues.  (Four waves of 128 x 128, one per SIMD, read a
+// third fewer fragment bytes per MFMA: with this file's kernel instantiated that way -- MT = 8 -- the plain
+// product is 1-2 % faster and the residual and q/k epilogues, which a lone wave cannot overlap with anything,
+// 3-10 % slower; a whole Flux step measures the same either way.)
 // ------------------------------------------------------------------------------------------
 constexpr int kEpiBytesPerWave = 64 * kEpiPitch;  // 17 408; eight of them fit the operand stages
 
+template <int MT>
 struct EpiOperands {
-  u32x2 bias[4][4];  // [tn][rq]: 4 consecutive bf16 at n = tn*32 + 8*rq + 4*g
-  float sc[2];       // [tm]: a_scale[m] * w_scale
+  u32x2 bias[8];  // [tn]: 4 consecutive bf16 at n = tn*16 + 4*q
+  float sc[MT];   // [tm]: a_scale[m] * w_scale, m = tm*16 + i
 };
 
 // QK: the wave's 128 columns are one head of a packed qkv projection; q and k heads get the per-head RMSNorm and
 // the RoPE rotation (same helper and rounding points as rmsnorm_rope_qk_kernel, so the result is bit-identical to
 // that kernel run in place on the stored projection) between the LDS read-back and the global store: there the
 // 16 lanes of a DPP row hold one token's whole head row, 16 bytes each.
-template <bool RESID, bool QK>
-__device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4][2], const EpiOperands& e,
+// MT: 16-token accumulator columns of the wave (4 or 8); HB: which 64 tokens (four columns) of them this call
+// stores; m_base is the first of those 64 tokens.
+template <bool RESID, bool QK, int MT, int HB>
+__device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x4 (&acc)[8][MT], const EpiOperands<MT>& e,
                                               uint8_t* wave_lds, int n_base, int m_base, int lane) {
-  const int g = lane >> 5, li = lane & 31;
-  // One half (32 token rows = one accumulator column tm) at a time: scale, add bias, round, stage in LDS.  The
+  const int q = lane >> 4, i16 = lane & 15;
+  // One half (32 token rows = two accumulator columns tm) at a time: scale, add bias, round, stage in LDS.  The
   // global stores of the first half are then in flight while the second half is converted.
-  auto stage_half = [&](int tm) {
-    const float sc = e.sc[tm];
-    uint8_t* lrow = wave_lds + (tm * 32 + li) * kEpiPitch;
+  auto stage_half = [&](int h) {
 #pragma unroll
-    for (int tn = 0; tn < 4; ++tn) {
+    for (int tmi = 0; tmi < 2; ++tmi) {
+      const int tl = 2 * h + tmi, tm = HB * 4 + tl;
+      const float sc = e.sc[tm];
+      uint8_t* lrow = wave_lds + (tl * 16 + i16) * kEpiPitch;
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        const int nl = tn * 32 + 8 * rq + 4 * g;
-        const u32x2 bw = e.bias[tn][rq];
+      for (int tn = 0; tn < 8; ++tn) {
+        const int nl = tn * 16 + 4 * q;
+        const u32x2 bw = e.bias[tn];
         u32x2 o;
-        o.x = pack_bf16x2(acc[tn][tm][4 * rq + 0] * sc + bf16_lo(bw.x),
-                          acc[tn][tm][4 * rq + 1] * sc + bf16_hi(bw.x));
-        o.y = pack_bf16x2(acc[tn][tm][4 * rq + 2] * sc + bf16_lo(bw.y),
-                          acc[tn][tm][4 * rq + 3] * sc + bf16_hi(bw.y));
+        o.x = pack_bf16x2(acc[tn][tm][0] * sc + bf16_lo(bw.x), acc[tn][tm][1] * sc + bf16_hi(bw.x));
+        o.y = pack_bf16x2(acc[tn][tm][2] * sc + bf16_lo(bw.y), acc[tn][tm][3] * sc + bf16_hi(bw.y));
         *reinterpret_cast<u32x2*>(lrow + nl * 2) = o;
       }
     }
@@ -336,15 +342,15 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
   };
   const bool interior = m_base + 64 <= p.M && n_base + 128 <= p.N;  // wave-uniform
   if (RESID && interior) {
-    u32x4 rva[8], rvb[8];
+    u32x4 rv[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) rva[u] = *reinterpret_cast<const u32x4*>(res_lane + u * res_step);
+    for (int u = 0; u < 8; ++u) rv[u] = *reinterpret_cast<const u32x4*>(res_lane + u * res_step);
     stage_half(0);
+    rows8_prefetched(0, rv);
 #pragma unroll
-    for (int u = 0; u < 8; ++u) rvb[u] = *reinterpret_cast<const u32x4*>(res_lane + (8 + u) * res_step);
-    rows8_prefetched(0, rva);
+    for (int u = 0; u < 8; ++u) rv[u] = *reinterpret_cast<const u32x4*>(res_lane + (8 + u) * res_step);
     stage_half(1);
-    rows8_prefetched(8, rvb);
+    rows8_prefetched(8, rv);
     return;
   }
 #pragma unroll
@@ -360,11 +366,18 @@ __device__ __forceinline__ void store_ct_lds(const GemmArgs& p, f32x16 (&acc)[4]
 // s_waitcnt immediate for vmcnt(vm) and lgkmcnt(lgkm) (15 = do not wait), expcnt left alone
 constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (lgkm << 8); }
 
-// WM = waves along m: 4 (256 x 256 tile, eight waves) or 2 (256 (n) x 128 (m) tile, four waves, for problems with
-// so few 256 x 256 tiles that half the compute units would idle; same wave tile, same K order, same bits).
-template <bool RESID, bool QK, int WM = 4>
+// WM = waves along m, MT = 16-token MFMA columns per wave; the wave tile is 128 (n) x 16 MT (m):
+//   WM 4, MT 4: 256 x 256 tile, eight waves of 128 x 64, two per SIMD;
+//   WM 2, MT 4: 256 (n) x 128 (m) tile, four waves, for problems with so few 256 x 256 tiles that half the compute
+//               units would idle.
+// (WM 2, MT 8 -- four waves of 128 x 128 on a 256 x 256 tile, accumulators in 256 AccVGPRs -- compiles and passes
+// the same tests; it is not instantiated, see above.)
+// Same K order in every form, so a row's bits do not depend on which of them computed it.
+template <bool RESID, bool QK, int WM = 4, int MT = 4>
 __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
-  constexpr int PW = 16 / WM;  // 1 KiB pieces of a W unit (256 rows) per wave; an A unit (64 WM rows) gives 4
+  constexpr int PW = 16 / WM;  // 1 KiB pieces of a W unit (256 rows) per wave
+  constexpr int PA = MT;       // 1 KiB pieces of an A unit (32 WM MT rows) per wave
+  constexpr int TM = WM * MT * 16;  // token rows of the tile
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   // Both problems' arguments are fetched together with the tile counts, in one round of scalar loads, and the
   // selected set is pinned in front of the early exit: left alone, the compiler sinks the argument loads below
@@ -383,12 +396,11 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
   const int lane = tid & 63;
   const int wave = tid >> 6;            // 0..2 WM - 1
   const int wn = wave / WM, wm = wave % WM;
-  const int g = lane >> 5, li = lane & 31;
-  const int m0 = tm * (64 * WM), n0 = tn * BN;
+  const int m0 = tm * TM, n0 = tn * BN;
 
   // async loads: per unit a wave issues one instruction per 8 rows of its share
   const int ld_r = lane >> 3, ld_p = lane & 7;
-  uint32_t w_off[PW], a_off[4];
+  uint32_t w_off[PW], a_off[PA];
 #pragma unroll
   for (int i = 0; i < PW; ++i) {
     const int row = (wave * PW + i) * 8 + ld_r;
@@ -396,18 +408,17 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
     w_off[i] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.ldw + c * 16;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = (wave * 4 + i) * 8 + ld_r;
+  for (int i = 0; i < PA; ++i) {
+    const int row = (wave * PA + i) * 8 + ld_r;
     const int c = ld_p ^ ((row >> 1) & 7);
     a_off[i] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.lda + c * 16;
   }
   const uint8_t* w_base = p.w + (int64_t)n0 * p.ldw;
   const uint8_t* a_base = p.a + (int64_t)m0 * p.lda;
-  const int nk = p.K / SK;
-  const int nu = nk / 2;
+  const int nu = p.K / UK;
   // The async loads are issued as assembly in the scalar-base + 32-bit-lane-offset form: the builtin takes a
-  // 64-bit per-lane address, and eight of those (plus their increments) are sixteen registers this kernel,
-  // at 256 per wave, does not have.  M0 carries the LDS destination; nothing else here uses M0.
+  // 64-bit per-lane address, and eight of those (plus their increments) are sixteen registers the eight-wave
+  // form, at 256 per wave, does not have.  M0 carries the LDS destination; nothing else here uses M0.
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)smem;
 #pragma clang diagnostic push
@@ -415,7 +426,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
   auto issue_load = [&](int j, int op, int i) {
     const int slot = (2 * j + op) % NSLOT;
     j = min(j, nu - 1);
-    const uint32_t dst = lds0 + slot * kUnitBytes + (wave_u * (op ? 4 : PW) + i) * 1024;
+    const uint32_t dst = lds0 + slot * kUnitBytes + (wave_u * (op ? PA : PW) + i) * 1024;
     const uint8_t* ub = (op ? a_base : w_base) + (int64_t)j * UK;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
@@ -424,105 +435,126 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
   };
 #pragma clang diagnostic pop
 
-  // Fragments: 4 W tiles + 2 A tiles, two 16-byte halves each = 12 LDS reads per step.  W tile i feeds MFMAs
-  // 2i and 2i+1 only, so the next step's W tile i is read into the SAME registers right after MFMA 2i+1 (seven
-  // MFMAs before its use); only the A fragments, which every MFMA of a step reads, are double-buffered.  That
-  // is 64 fragment registers instead of 96, which is what lets 128 accumulators fit in 256 registers.
-  const int w_row = wn * 128 + li;
-  const int a_row = wm * 64 + li;
-  i32x4 fw[4][2];
-  i32x4 fa[2][2][2];  // [buffer][tile][half]
-  // read addresses: one lane constant per (step parity, half) and operand; the tile adds 32 rows = 4096 bytes
-  // (the swizzle of row + 32t equals that of row) and the ring slot adds a scalar
-  uint32_t w_la[2][2], a_la[2][2];
+  // Operand fragments of v_mfma_f32_16x16x128_f8f6f4: lane (q = lane / 16, i = lane % 16) holds the 32 K-bytes
+  // [32q, 32q + 32) of row i of a 16-row tile, i.e. chunks 2q and 2q + 1 of a 128-byte unit row: one MFMA consumes
+  // a whole unit row of either operand.  A wave's tile is 8 W tiles x MT A tiles = 8 MT MFMAs per unit.  W tile i
+  // feeds MFMAs i MT .. i MT + MT - 1 only, so W fragments live in a ring of four register octets and are read
+  // three tiles ahead of their use; the A fragments, which every W tile meets, are double-buffered per unit.
+  const int q16 = lane >> 4, i16 = lane & 15;
+  const int w_row = wn * 128 + i16;
+  const int a_row = wm * (MT * 16) + i16;
+  i32x4 wr[4][2];      // [ring slot][half]
+  i32x4 ar[2][MT][2];  // [buffer][tile][half]
+  // Read addresses: a lane constant per half and operand (a tile adds 16 rows = 2048 bytes as an immediate: the
+  // swizzle of row + 16t equals that of row) plus the ring slot of the unit.  The sums live in registers that are
+  // re-pointed once per unit -- wa[k]: W of units of parity k (the unit being computed and the next one alternate
+  // between the two), aa: A of the next unit -- instead of being formed at each of a unit's 16 + 2 MT reads.
+  uint32_t w_la[2], a_la[2], wa[2][2], aa[2];
 #pragma unroll
-  for (int par = 0; par < 2; ++par)
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      w_la[par][half] = (uint32_t)unit_off(w_row, par * 4 + g * 2 + half);
-      a_la[par][half] = (uint32_t)unit_off(a_row, par * 4 + g * 2 + half);
-    }
-  auto read_w = [&](int j, int par, int t, int half) {   // W fragment (tile t) of MFMA step 2j + par
+  for (int half = 0; half < 2; ++half) {
+    w_la[half] = (uint32_t)unit_off(w_row, q16 * 2 + half);
+    a_la[half] = (uint32_t)unit_off(a_row, q16 * 2 + half);
+  }
+  auto point_w = [&](int k, int j) {  // wa[k] -> W of unit j
     uint32_t slot_off = (uint32_t)(((2 * j) % NSLOT) * kUnitBytes);
-    asm volatile("" : "+s"(slot_off));  // added at the read, from a scalar: not a register per combination
-    fw[t][half] = *reinterpret_cast<const i32x4*>(smem + (slot_off + w_la[par][half]) + t * 4096);
+    asm volatile("" : "+s"(slot_off));
+    wa[k][0] = w_la[0] + slot_off;
+    wa[k][1] = w_la[1] + slot_off;
   };
-  auto read_a = [&](int buf, int j, int par, int t, int half) {
+  auto point_a = [&](int j) {  // aa -> A of unit j
     uint32_t slot_off = (uint32_t)(((2 * j + 1) % NSLOT) * kUnitBytes);
     asm volatile("" : "+s"(slot_off));
-    fa[buf][t][half] = *reinterpret_cast<const i32x4*>(smem + (slot_off + a_la[par][half]) + t * 4096);
+    aa[0] = a_la[0] + slot_off;
+    aa[1] = a_la[1] + slot_off;
+  };
+  auto read_w = [&](int k, int tile, int half) {   // W tile `tile` (0..7) of the unit wa[k] points at
+    wr[tile & 3][half] = *reinterpret_cast<const i32x4*>(smem + wa[k][half] + tile * 2048);
+  };
+  auto read_a = [&](int buf, int tile, int half) {
+    ar[buf][tile][half] = *reinterpret_cast<const i32x4*>(smem + aa[half] + tile * 2048);
   };
 
-  f32x16 acc[4][2];
+  f32x4 acc[8][MT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < MT; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-  auto mfma_one = [&](int buf, int idx) {   // idx 0..7: W tile idx/2, A tile idx%2
-    const int i = idx >> 1, j = idx & 1;
-    const i32x8 vw = {fw[i][0].x, fw[i][0].y, fw[i][0].z, fw[i][0].w, fw[i][1].x, fw[i][1].y, fw[i][1].z, fw[i][1].w};
-    const i32x8 va = {fa[buf][j][0].x, fa[buf][j][0].y, fa[buf][j][0].z, fa[buf][j][0].w,
-                      fa[buf][j][1].x, fa[buf][j][1].y, fa[buf][j][1].z, fa[buf][j][1].w};
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vw, va, acc[i][j], 0, 0, 0, 0, 0, 0);
+  auto mfma_one = [&](int buf, int i, int t) {   // W tile i x A tile t
+    const i32x4 w0 = wr[i & 3][0], w1 = wr[i & 3][1], a0 = ar[buf][t][0], a1 = ar[buf][t][1];
+    const i32x8 vw = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+    const i32x8 va = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    acc[i][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vw, va, acc[i][t], 0, 0, 0, 0, 0, 0);
   };
 
   // Operands of the epilogue.  Columns >= N and rows >= M are never stored, so their addresses are clamped
   // instead of predicated (a lane-predicated load is not batched with its neighbours).
-  EpiOperands epi;
+  EpiOperands<MT> epi;
   float w_scale_raw = 1.0f;
   auto load_epi = [&]() {  // loads only: whatever uses a loaded value would wait for it on the spot
-    const int n_base = n0 + wn * 128, m_base = m0 + wm * 64;
+    const int n_base = n0 + wn * 128, m_base = m0 + wm * (MT * 16);
     if (p.w_scale) w_scale_raw = *p.w_scale;
     if (p.bias) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int rq = 0; rq < 4; ++rq)
-          epi.bias[t][rq] = *reinterpret_cast<const u32x2*>(
-              p.bias + min(n_base + t * 32 + 8 * rq + 4 * g, p.N - 4));
+      for (int t = 0; t < 8; ++t)
+        epi.bias[t] = *reinterpret_cast<const u32x2*>(p.bias + min(n_base + t * 16 + 4 * q16, p.N - 4));
     } else {
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int rq = 0; rq < 4; ++rq) epi.bias[t][rq] = u32x2{0, 0};
+      for (int t = 0; t < 8; ++t) epi.bias[t] = u32x2{0, 0};
     }
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-      epi.sc[t] = p.a_scale ? p.a_scale[min(m_base + t * 32 + li, p.M - 1)] : 1.0f;
+    for (int t = 0; t < MT; ++t)
+      epi.sc[t] = p.a_scale ? p.a_scale[min(m_base + t * 16 + i16, p.M - 1)] : 1.0f;
   };
 
-  // One step = 8 MFMAs per wave; the fragments of step 2j + par sit in fw and fa[par].  Between the MFMAs the
-  // wave reads the 12 fragments of the next step and issues its async loads of unit j + 2 (the even step the
-  // PW pieces of W, the odd step the 4 of A).  `loads` = false for
-  // the last two units (nothing is left to fetch; the odd step then waits for everything in flight);
-  // `last` = true for the very last step: no next fragments, and the registers they would occupy take the
-  // epilogue's operands instead, whose latency the remaining MFMAs cover.
-  auto step = [&](int j, int par, bool loads, bool last) {
-    if (par) {
-      if (loads)
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(PW, 0));  // all but the W pieces the even step just issued; lgkmcnt(0)
-      else
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));   // vmcnt(0) lgkmcnt(0)
-      __builtin_amdgcn_s_barrier();
-    } else {
-      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-    }
+  // One unit = 128 bytes of K = 8 MT MFMAs per wave (slot s: W tile s / MT, A tile s % MT); the A fragments of
+  // unit j sit in ar[buf], its first three W tiles in the ring, wa[par] points at its W slot and wa[par ^ 1] at the
+  // next unit's.  Between the MFMAs the wave reads W tile s / MT + 3 (in the first two slots of a tile, one half
+  // each), which from slot 5 MT on is a tile of unit j + 1, reads the A fragments of unit j + 1 into the other
+  // buffer (2 MT slots from 5 MT + 2 on), issues its async loads of W unit j + 2 (slots below 4 MT) and of A unit
+  // j + 2 (after slot 5 MT).  Slot 5 MT opens with the unit's one synchronisation point: every load but the W pieces
+  // just issued has landed (unit j + 1 is complete), every wave has finished reading unit j (its last W tile was
+  // read in slots 4 MT and 4 MT + 1), so unit j's two ring slots can be overwritten -- A unit j + 2 takes the one
+  // W unit j had, W unit j + 3 (a unit later) the one A unit j had.
+  // `loads` = false for the last two units (nothing is left to fetch); `last` = true for the very last: no next
+  // unit to read from, and the registers its fragments would occupy take the epilogue's operands instead.
+  constexpr int NS = 8 * MT, kSync = 5 * MT;
+  auto unit = [&](int j, int par, bool loads, bool last) {
+    const int buf = par;
 #pragma unroll
-    for (int idx = 0; idx < 8; ++idx) {
-      mfma_one(par, idx);
-      if (last) {
-        if (idx == 0) load_epi();
-      } else if (idx & 1) {  // W tile idx/2 has been read for the last time in this step
-        read_w(j + par, par ^ 1, idx >> 1, 0);
-        read_w(j + par, par ^ 1, idx >> 1, 1);
-      } else {
-        read_a(par ^ 1, j + par, par ^ 1, idx >> 2, (idx >> 1) & 1);
-        if (loads && (par || PW == 4)) issue_load(j + 2, par, idx >> 1);
+    for (int s = 0; s < NS; ++s) {
+      const int i = s / MT, t = s % MT;
+      if (s == kSync) {
+        if (loads)
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(PW, 0));  // all but the W pieces of this unit; lgkmcnt(0)
+        else
+          __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));   // vmcnt(0) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        if (!last) {
+          point_w(par, j + 2);  // this unit's W slot has been read for the last time: on to the unit after next
+          point_a(j + 1);
+        }
       }
-      if (PW == 8 && !par && loads && !last) issue_load(j + 2, 0, idx);  // eight W pieces: one per slot
+      mfma_one(buf, i, t);
+      if (t < 2) {
+        const int tile = i + 3;
+        if (tile < 8)
+          read_w(par, tile, t);
+        else if (!last)
+          read_w(par ^ 1, tile - 8, t);
+      }
+      if (last) {
+        if (s == 6 * MT) load_epi();  // the W ring is down to its last two tiles: their neighbours take the operands
+      } else {
+        if (s >= kSync + 2 && s < kSync + 2 + 2 * MT) read_a(buf ^ 1, (s - kSync - 2) >> 1, (s - kSync - 2) & 1);
+        if (loads) {
+          constexpr int kWStride = 4 * MT / PW;
+          if (s < 4 * MT && (s % kWStride) == kWStride - 1) issue_load(j + 2, 0, s / kWStride);
+          if (s > kSync && (s - kSync - 1) % 3 == 0 && (s - kSync - 1) / 3 < PA) issue_load(j + 2, 1, (s - kSync - 1) / 3);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -530,37 +562,66 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int i = 0; i < ((u & 1) ? 4 : PW); ++i) issue_load(u >> 1, u & 1, i);
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(PW + 4, 15));  // all but W and A unit 1: W and A unit 0 have landed
+    for (int i = 0; i < ((u & 1) ? PA : PW); ++i) issue_load(u >> 1, u & 1, i);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(PW + PA, 15));  // all but W and A unit 1: W and A unit 0 have landed
   __builtin_amdgcn_s_barrier();
+  // Parity of unit j: (j + nu) % 2, so that the last unit always has parity 1 and the one before it parity 0
+  // whatever the unit count; it selects the A buffer and which of wa[] points at the unit.
+  point_a(0);
+  if (nu & 1) {
+    point_w(1, 0);
+    point_w(0, 1);
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    read_w(0, 0, t, 0);
-    read_w(0, 0, t, 1);
-  }
+    for (int t = 0; t < 3; ++t) {
+      read_w(1, t, 0);
+      read_w(1, t, 1);
+    }
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    read_a(0, 0, 0, t, 0);
-    read_a(0, 0, 0, t, 1);
+    for (int t = 0; t < MT; ++t) {
+      read_a(1, t, 0);
+      read_a(1, t, 1);
+    }
+  } else {
+    point_w(0, 0);
+    point_w(1, 1);
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      read_w(0, t, 0);
+      read_w(0, t, 1);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      read_a(0, t, 0);
+      read_a(0, t, 1);
+    }
   }
 
-  for (int j = 0; j < nu - 2; ++j) {
-    step(j, 0, true, false);
-    step(j, 1, true, false);
+  {
+    int j = 0;
+    const int n_loading = nu >= 2 ? nu - 2 : 0;  // units that still have loads to issue
+    if (n_loading & 1) {
+      unit(0, 1, true, false);
+      j = 1;
+    }
+    for (; j < n_loading; j += 2) {
+      unit(j, 0, true, false);
+      unit(j + 1, 1, true, false);
+    }
+    if (nu >= 2) unit(nu - 2, 0, false, false);
+    unit(nu - 1, 1, false, true);
   }
-  if (nu >= 2) {
-    step(nu - 2, 0, false, false);
-    step(nu - 2, 1, false, false);
-  }
-  step(nu - 1, 0, false, false);
-  step(nu - 1, 1, false, true);
-  // No barrier in front of the epilogue: the last step's own barrier came after every wave's final fragment
-  // reads (lgkmcnt(0)) and after every async load had landed (vmcnt(0)), and the last step touches neither, so
-  // the ring is dead from there on and a wave may overwrite its private staging region as soon as its own MFMAs
-  // are issued -- the two waves of a SIMD then overlap one's conversion with the other's last MFMAs.
-  epi.sc[0] *= w_scale_raw;
-  epi.sc[1] *= w_scale_raw;
-  store_ct_lds<RESID, QK>(p, acc, epi, smem + wave * kEpiBytesPerWave, n0 + wn * 128, m0 + wm * 64, lane);
+  // No barrier in front of the epilogue: the last unit's synchronisation point came after every wave's final
+  // fragment reads and after every async load had landed, so the ring is dead from there on and a wave may
+  // overwrite its private staging region as soon as its own MFMAs are issued.
+  // (compiler-only fence: without it the epilogue's residual loads are hoisted into the last unit, where every
+  // register is taken, and the accumulators they displace are spilled)
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int t = 0; t < MT; ++t) epi.sc[t] *= w_scale_raw;
+  uint8_t* const stage = smem + wave * kEpiBytesPerWave;
+  store_ct_lds<RESID, QK, MT, 0>(p, acc, epi, stage, n0 + wn * 128, m0 + wm * (MT * 16), lane);
+  if constexpr (MT == 8)
+    store_ct_lds<RESID, QK, MT, 1>(p, acc, epi, stage, n0 + wn * 128, m0 + wm * (MT * 16) + 64, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -721,20 +782,15 @@ static int gemm_set_attributes() {
   using namespace dsx;
   static PerDeviceOnce once;
   return per_device_once(once, [](int) {
-    if (hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, false, 2>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_kernel<true, false, 2>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_kernel<false, true, 2>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes) != hipSuccess)
+    const void* kernels[] = {
+        (const void*)fp8_gemm_kernel<false, false, 4, 4>, (const void*)fp8_gemm_kernel<true, false, 4, 4>,
+        (const void*)fp8_gemm_kernel<false, true, 4, 4>,  (const void*)fp8_gemm_kernel<false, false, 2, 4>,
+        (const void*)fp8_gemm_kernel<true, false, 2, 4>,  (const void*)fp8_gemm_kernel<false, true, 2, 4>};
+    for (const void* k : kernels)
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess)
+        return (int)DSX_ELAUNCH;
+    if (hipFuncSetAttribute((const void*)fp8_gemm_ragged_k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kStageBytes) != hipSuccess)
       return (int)DSX_ELAUNCH;
     return (int)DSX_OK;
   });
@@ -771,20 +827,20 @@ static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStre
     q.total = q.total0 + (p1 ? q.p[1].tiles_m * p1->tiles_n : 0);
     const int grid = ((q.total + 7) / 8) * 8;
     if (p0.resid)
-      fp8_gemm_kernel<true, false, 2><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+      fp8_gemm_kernel<true, false, 2, 4><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
     else if (p0.qk_heads > 0)
-      fp8_gemm_kernel<false, true, 2><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+      fp8_gemm_kernel<false, true, 2, 4><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
     else
-      fp8_gemm_kernel<false, false, 2><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+      fp8_gemm_kernel<false, false, 2, 4><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
     return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
   }
   const int grid = ((q.total + 7) / 8) * 8;
   if (p0.resid)
-    fp8_gemm_kernel<true, false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<true, false, 4, 4><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   else if (p0.qk_heads > 0)
-    fp8_gemm_kernel<false, true><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<false, true, 4, 4><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   else
-    fp8_gemm_kernel<false, false><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+    fp8_gemm_kernel<false, false, 4, 4><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 

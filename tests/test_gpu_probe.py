@@ -25,7 +25,10 @@ def test_every_probe_kind_runs_and_counts_its_flops(dev):
         flops = ctypes.c_int64(0)
         rc = lib.dsx_mfma_ceiling_probe(kind, bits.data_ptr(), 50, 7, sink.data_ptr(), ctypes.byref(flops), stream)
         assert rc == _lib.DSX_OK, (kind, rc)
-        # 7 workgroups x 4 wavefronts x 50 iterations x 4 MFMAs
-        assert flops.value == 7 * 4 * 50 * 4 * per_mfma[kind & 3]
+        # 7 workgroups x 4 wavefronts x 50 rounds x (4 MFMAs of a 32x32 shape, 8 of a 16x16 shape)
+        assert flops.value == 7 * 4 * 50 * (8 if (kind & 3) >= 2 else 4) * per_mfma[kind & 3]
     torch.cuda.synchronize()
     assert sink.item() == 0.0
+    # the caps that keep one call from occupying the device for minutes
+    assert lib.dsx_mfma_ceiling_probe(0, bits.data_ptr(), (1 << 22) + 1, 7, sink.data_ptr(), None, stream) == _lib.DSX_EBADSHAPE
+    assert lib.dsx_mfma_ceiling_probe(0, bits.data_ptr(), 50, (1 << 14) + 1, sink.data_ptr(), None, stream) == _lib.DSX_EBADSHAPE
