@@ -11,6 +11,9 @@ namespace dsx {
 int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_bytes, hipStream_t stream);
 // Scratch bytes with which launch_attn_plain would split (0 when it would not).
 int64_t attn_plain_workspace_bytes(const dsx_attn_params& p);
+// The same attention on the 16x16x32 MFMA shape (attn_plain16.hip), for launches of several full rounds of
+// workgroups; whole units only (no key split, no fused q pre-processing).  launch_attn_plain decides.
+int launch_attn_plain16(const dsx_attn_params& p, int64_t units, hipStream_t stream);
 }  // namespace dsx
 
 #ifdef __HIPCC__

@@ -1,17 +1,14 @@
-// Flash attention forward for gfx950 without fused k pre-processing (k already normalised and rotated; q may
-// still need it): head dim 128, bf16 operands, fp32 online softmax.
+// Flash attention forward for gfx950 without fused pre-processing (q and k already normalised
+// and rotated): head dim 128, bf16 operands, fp32 online softmax.
 //
-// MFMA formulation: S^T = K Q^T and O^T += V^T P^T on v_mfma_f32_16x16x32_bf16 (on N(0,1) operands, where the chip
-// runs at its power limit, a bare stream of this shape sustains 12 % more than one of v_mfma_f32_32x32x16_bf16:
-// 2.08 against 1.86 PFLOP/s).  A wave owns 32 queries = two 16-query MFMA columns; lane (q = lane / 16,
-// i = lane % 16) holds, for each of its two queries 16t + i, the scores of keys 16kt + 4q .. 4q + 3 of every
-// 16-key tile kt: a query's row is spread over the four lanes i, i + 16, i + 32, i + 48, so the exponentials are
-// lane-local and only row maxima / row sums cross lanes (two permlane swaps).  Packed to bf16, the scores of two
-// neighbouring key tiles are exactly the B operand of the second product (K extent 32 keys): no LDS round trip.
+// MFMA formulation as in attn_fwd.hip (S^T = K Q^T, O^T += V^T P^T, one query per lane, so the
+// softmax statistics are lane-local apart from one exchange between the two half-waves).
 //
-// Work split: one workgroup = 8 waves = 256 consecutive queries of one (batch, head); every wave needs ~240 VGPRs,
-// so two waves share a SIMD and one workgroup fills a CU.  While one wave of a SIMD works through
-// exp2/convert/row-sum on the VALU, the other's MFMAs can keep the matrix pipe busy.
+// Work split: one workgroup = 8 waves = 256 consecutive queries of one (batch, head); every wave
+// owns 32 queries and needs ~230 VGPRs, so two waves share a SIMD and one workgroup fills a CU.
+// While one wave of a SIMD works through exp2/convert/row-sum on the VALU, the other's MFMAs can
+// keep the matrix pipe busy.  That costs one LDS operand read per MFMA, which the 256 B/clk LDS of
+// CDNA4 carries at a quarter load.
 //
 //  * K and V blocks (64 keys) go HBM/L2 -> LDS with global_load_lds_dwordx4, four stages deep,
 //    both stored row-major [key][128 d].  No staging registers, no transposing stores.
@@ -25,9 +22,8 @@
 //    128*scale*log2(e) ~ 16.  Moving the reference rescales O and l, so the result is exact
 //    softmax in every case.
 //
-// LDS swizzles: K rows (256 B): 16-byte chunk c of key r at c ^ (r & 15)        (ds_read_b128 by 16 rows x 4 chunks);
-//               V rows (256 B): chunk c of key r at c ^ ((r & 7) << 1)          (transposing 8-byte reads of
-//                                                                                16 keys x 32 bytes).
+// LDS swizzles: K rows (256 B): 16-byte chunk c of key r at c ^ (r & 15)  (ds_read_b128 by 32 rows);
+//               V rows (256 B): chunk c of key r at c ^ ((r & 3) << 2)    (transposing 8-byte reads).
 #include <algorithm>
 
 #include "attn_internal.h"
@@ -50,19 +46,13 @@ typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 typedef short v4i16 __attribute__((ext_vector_type(4)));
 
-// Reductions over the four lanes i, i + 16, i + 32, i + 48 that share a query.  permlane16_swap(v, v) returns
-// (rows 0 0 2 2, rows 1 1 3 3) of v, permlane32_swap(v, v) (lower half twice, upper half twice).
-__device__ __forceinline__ float quad_max(float v) {
-  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+__device__ __forceinline__ float pair_max(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
-__device__ __forceinline__ float quad_sum(float v) {
-  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  const float m = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
-  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+__device__ __forceinline__ float pair_sum(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 
@@ -78,22 +68,24 @@ struct AttnSplit {
   float* slots;
   int device_bound;  // the kernel reads p.qk_norm2_max and returns at once when the other variant is the one to run
 };
-constexpr int kSlotOFloats = QB * HD;               // O part: [dt][t][wave][lane][4]
+constexpr int kSlotOFloats = QB * HD;               // O part: [dt][rq][wave][g][j][4]
 constexpr int kSlotFloats = kSlotOFloats + 2 * QB;  // + row sums, + references
 
-// normalised output of one lane for one of its two queries: query `row`, d = dt*16 + 4q + 0..3 per dt
-__device__ __forceinline__ void store_output(const dsx_attn_params& p, int b, int h, int64_t row, int q4,
-                                             const f32x4 (&oacc)[8][2], int t, float inv) {
+// normalised output of one lane: query `row`, d = dt*32 + 8*rq + 4g + 0..3 per (dt, rq)
+__device__ __forceinline__ void store_output(const dsx_attn_params& p, int b, int h, int64_t row, int g,
+                                             const f32x16 (&oacc)[4], float inv) {
   const int seg = row >= p.sq[0] ? 1 : 0;
   uint16_t* dst = (uint16_t*)p.o[seg] + (int64_t)b * p.o_sb[seg] + (int64_t)h * p.o_sh[seg] +
                   (row - (seg ? p.sq[0] : 0)) * p.o_ss[seg];
 #pragma unroll
-  for (int dt = 0; dt < 8; ++dt) {
-    u32x2 w;
-    w.x = pack_bf16x2(oacc[dt][t][0] * inv, oacc[dt][t][1] * inv);
-    w.y = pack_bf16x2(oacc[dt][t][2] * inv, oacc[dt][t][3] * inv);
-    *reinterpret_cast<u32x2*>(dst + dt * 16 + 4 * q4) = w;
-  }
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      u32x2 w;
+      w.x = pack_bf16x2(oacc[dt][4 * rq + 0] * inv, oacc[dt][4 * rq + 1] * inv);
+      w.y = pack_bf16x2(oacc[dt][4 * rq + 2] * inv, oacc[dt][4 * rq + 3] * inv);
+      *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w;
+    }
 }
 
 // SCAN = false: the caller has bounded every |score| (log2 domain) by kRescaleThreshold, so the softmax
@@ -116,7 +108,7 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;  // 0..7
-  const int q4 = lane >> 4, i16 = lane & 15;
+  const int g = lane >> 5, li = lane & 31;
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of (batch, head,
   // query block) units so that the query blocks of one head share that head's K/V through ONE L2
   // (with a plain 3-D grid every XCD ends up fetching every head's K and V).
@@ -185,7 +177,7 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
       const int seg = key >= p.skv[0] ? 1 : 0;
       const int64_t lrow = key - (seg ? p.skv[0] : 0);
       kp[i] = kbase[seg] + lrow * p.k_ss[seg] * 2 + ((ld_p ^ (row & 15)) << 4);
-      vp[i] = vbase[seg] + lrow * p.v_ss[seg] * 2 + ((ld_p ^ ((row & 7) << 1)) << 4);
+      vp[i] = vbase[seg] + lrow * p.v_ss[seg] * 2 + ((ld_p ^ ((row & 3) << 2)) << 4);
     }
   };
   // uniform per-block pointer strides (bytes) of both segments, and the key counts as 32-bit scalars (the
@@ -244,19 +236,17 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
   if (kb_begin + 2 < kb_end) advance_to(kb_begin + 2);
   issue_block(2);
 
-  // ---- Q fragments (B operand of S^T = K Q^T), pre-multiplied by scale*log2(e): qf[t][dc] = query 16t + i,
-  //      d = 32dc + 8q .. + 7
+  // ---- Q fragments (B operand of S^T = K Q^T), pre-multiplied by scale*log2(e)
   const float c = p.softmax_scale * kLog2e;
-  bf16x8 qf[2][4];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    int64_t row = q0 + t * 16 + i16;
+  bf16x8 qf[8];
+  {
+    int64_t row = q0 + li;
     if (row >= Sq) row = Sq - 1;
     const int seg = row >= p.sq[0] ? 1 : 0;
     const uint16_t* src = qbase[seg] + (row - (seg ? p.sq[0] : 0)) * p.q_ss[seg];
-    u32x4 raws[4];
+    u32x4 raws[8];
 #pragma unroll
-    for (int dc = 0; dc < 4; ++dc) raws[dc] = *reinterpret_cast<const u32x4*>(src + dc * 32 + q4 * 8);
+    for (int kc = 0; kc < 8; ++kc) raws[kc] = *reinterpret_cast<const u32x4*>(src + kc * 16 + g * 8);
     if (QPRE) {
       const uint16_t* nw = (const uint16_t*)p.q_norm_w[seg];
       const float* rope = p.rope ? p.rope + (int64_t)b * p.rope_sb + row * HD : nullptr;
@@ -264,56 +254,56 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
       if (nw) {
         float ss = 0.f;
 #pragma unroll
-        for (int dc = 0; dc < 4; ++dc) ss += sumsq_chunk(raws[dc]);
-        rrms = rsqrtf(quad_sum(ss) * (1.0f / HD) + p.norm_eps);
+        for (int kc = 0; kc < 8; ++kc) ss += sumsq_chunk(raws[kc]);
+        rrms = rsqrtf(pair_sum(ss) * (1.0f / HD) + p.norm_eps);
       }
 #pragma unroll
-      for (int dc = 0; dc < 4; ++dc)
-        raws[dc] = norm_rope_chunk(raws[dc], nw != nullptr, rrms, nw ? nw + dc * 32 + q4 * 8 : nullptr,
-                                   rope ? rope + dc * 32 + q4 * 8 : nullptr);
+      for (int kc = 0; kc < 8; ++kc)
+        raws[kc] = norm_rope_chunk(raws[kc], nw != nullptr, rrms, nw ? nw + kc * 16 + g * 8 : nullptr,
+                                   rope ? rope + kc * 16 + g * 8 : nullptr);
     }
 #pragma unroll
-    for (int dc = 0; dc < 4; ++dc) {
-      const u32x4 raw = raws[dc];
+    for (int kc = 0; kc < 8; ++kc) {
+      const u32x4 raw = raws[kc];
       u32x4 sc;
       sc.x = pack_bf16x2(bf16_lo(raw.x) * c, bf16_hi(raw.x) * c);
       sc.y = pack_bf16x2(bf16_lo(raw.y) * c, bf16_hi(raw.y) * c);
       sc.z = pack_bf16x2(bf16_lo(raw.z) * c, bf16_hi(raw.z) * c);
       sc.w = pack_bf16x2(bf16_lo(raw.w) * c, bf16_hi(raw.w) * c);
-      qf[t][dc] = __builtin_bit_cast(bf16x8, sc);
+      qf[kc] = __builtin_bit_cast(bf16x8, sc);
     }
   }
 
-  f32x4 oacc[8][2];  // [d tile][query column]: lane (q, i): query 16t + i, d = 16dt + 4q .. + 3
+  f32x16 oacc[4];
 #pragma unroll
-  for (int dt = 0; dt < 8; ++dt)
+  for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-    for (int t = 0; t < 2; ++t) oacc[dt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_ref[2] = {0.f, 0.f};  // softmax reference of the lane's two queries (log2 domain)
-  bool any_ref = false;         // wave-uniform: some lane of this wave has a reference != 0
-  float l_run[2] = {0.f, 0.f};
+    for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+  float m_ref = 0.f;     // softmax reference of the lane's query (log2 domain)
+  bool any_ref = false;  // wave-uniform: some lane of this wave has m_ref != 0
+  float l_run = 0.f;
 
-  // transposing V reads: a 16-lane group q fetches keys 4q .. 4q + 3 of a 16-key half x 16 d; source lane j
-  // of the group points at key 4q + j/4, d bytes 8 (j % 4) of the 32-byte piece of d tile dt
-  const int tr_key = 4 * q4 + (i16 >> 2);
-  const int tr_dbyte = (i16 & 3) * 8;
-  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  // transposing V reads: source-lane role of this lane inside its 16-lane group
+  const int grp = lane >> 4, j16 = lane & 15;
+  const int tr_key = ((grp >> 1) << 2) + (j16 >> 2);    // 4*g of the receiving lanes + key within the quad
+  const int tr_dbyte = (grp & 1) * 32 + (j16 & 3) * 8;  // + dt*64, bytes within the 256-byte row
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // LDS read addresses = one lane-dependent VGPR per swizzle class + an immediate: the XOR
-  // swizzles only permute the 16-byte chunk (K) / 32-byte piece (V) index by lane-constant bits.
-  //   K fragment (kt, dc): key 16kt + i, chunk (4dc + q) ^ i
-  //   V^T datum (key 32c + 16hi + tr_key, dt): 32-byte piece dt ^ (tr_key & 7), byte tr_dbyte within
-  uint32_t lane_k[4], lane_v[8];
+  // swizzles only permute the 16-byte chunk (K) / 64-byte group (V) index by lane-constant bits.
+  //   K fragment (kt, kc): key kt*32 + li, chunk (2kc+g) ^ (li & 15)
+  //   V^T datum (key0 + 32kt + 16ch + 8hi, dt): 64-byte group dt ^ (tr_key & 3), byte tr_dbyte within
+  uint32_t lane_k[8], lane_v[4];
 #pragma unroll
-  for (int dc = 0; dc < 4; ++dc) lane_k[dc] = i16 * 256 + (((4 * dc + q4) ^ i16) << 4);
+  for (int kc = 0; kc < 8; ++kc) lane_k[kc] = li * 256 + (((2 * kc + g) ^ (li & 15)) << 4);
 #pragma unroll
-  for (int dt = 0; dt < 8; ++dt)
-    lane_v[dt] = kStages * kTile + tr_key * 256 + ((dt ^ (tr_key & 7)) << 5) + tr_dbyte;
+  for (int dt = 0; dt < 4; ++dt)
+    lane_v[dt] = kStages * kTile + tr_key * 256 + ((dt ^ (tr_key & 3)) << 6) + tr_dbyte;
 
   // Software pipeline over 64-key blocks.  Interval kb (behind one workgroup barrier) runs
-  //   stage 1:  S(kb+1)^T = K(kb+1) Q^T, 32 MFMAs;
-  //   stage 2:  O^T += V(kb)^T P(kb)^T, 32 MFMAs;
-  // and the softmax of the wave's own scores is spread over the 64 MFMA slots so that neither stage asks
+  //   stage 1:  S(kb+1)^T = K(kb+1) Q^T, 16 MFMAs;
+  //   stage 2:  O^T += V(kb)^T P(kb)^T, 16 MFMAs;
+  // and the softmax of the wave's own scores is spread over the 32 MFMA slots so that neither stage asks
   // more of the VALU than the matrix pipe leaves time for when two waves share a SIMD: entries
   // kExpEarly.. of P(kb) = exp2(S(kb)) in stage 1, the block maximum of S(kb+1) in the first slots of
   // stage 2 (the PV MFMAs issued there cover the latency of the last QK MFMA), entries 0..kExpEarly-1 of
@@ -324,231 +314,202 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
   // Four stages of K and V: block kb+1 must have landed when interval kb starts, kb+2 is in flight,
   // kb+3 is issued into the stage block kb-1 has left.
   constexpr int kExpEarly = 12;  // even; entries of P(kb+1) produced during stage 2 of interval kb
-  constexpr int kAhead = 2;      // operand fragments in flight ahead of the MFMA pair that uses them
+  constexpr int kAhead = 2;      // operand fragments in flight ahead of the MFMA that uses them
   auto interval_head = [&](int kb) {
     __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4): only block kb+2 may still be in flight
     __builtin_amdgcn_s_barrier();
     if (__builtin_expect(kb + 3 < kb_end, 1)) advance_to(kb + 3);  // else: re-fetch the last block, nobody reads it
   };
-  // Scores of one block: s[kt][t][e] = query 16t + i against key 16kt + 4q + e.
-  // mask_tail masks the ragged tail of block `blk`; ref_scan subtracts the current reference and returns, for each of
-  // the lane's two queries, the maximum over the lane's own keys; ref_move shifts the references (rescaling O and l), which is needed only when
-  // a block maximum leaves the safe range.
-  auto mask_tail = [&](f32x4 (&s)[4][2], int blk) {
+  // Softmax reference.  mask_tail masks the ragged tail of block `blk`; ref_scan subtracts the current
+  // reference and returns the block maximum of the lane's query; ref_move shifts the reference (rescaling O and l), which
+  // is needed only when a block maximum leaves the safe range.
+  auto mask_tail = [&](f32x16 (&s)[2], int blk) {
     if (__builtin_expect((blk + 1) * KB > skv_all, 0)) {  // ragged tail of the key axis
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = blk * KB + kt * 16 + 4 * q4 + e;
-          if (key >= skv_all) s[kt][0][e] = s[kt][1][e] = -INFINITY;
+        for (int r = 0; r < 16; ++r) {
+          const int key = blk * KB + kt * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (key >= skv_all) s[kt][r] = -INFINITY;
         }
     }
   };
-  auto ref_scan = [&](f32x4 (&s)[4][2], float (&mx)[2]) {
+  auto ref_scan = [&](f32x16 (&s)[2], int blk) -> float {
+    if (__builtin_expect(any_ref, 0)) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      if (__builtin_expect(any_ref, 0)) {
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) s[kt][t][e] -= m_ref[t];
-      }
-      float m0 = max3(s[0][t][0], s[0][t][1], s[0][t][2]);
-      float m1 = max3(s[1][t][0], s[1][t][1], s[1][t][2]);
-      m0 = max3(m0, s[0][t][3], s[2][t][0]);
-      m1 = max3(m1, s[1][t][3], s[3][t][0]);
-      m0 = max3(m0, s[2][t][1], s[2][t][2]);
-      m1 = max3(m1, s[3][t][1], s[3][t][2]);
-      mx[t] = max3(m0, m1, fmaxf(s[2][t][3], s[3][t][3]));  // of the lane's own 16 keys: a quarter of the row
+        for (int r = 0; r < 16; ++r) s[kt][r] -= m_ref;
     }
+    float m0 = max3(s[0][0], s[0][1], s[0][2]);
+    float m1 = max3(s[1][0], s[1][1], s[1][2]);
+#pragma unroll
+    for (int r = 3; r < 15; r += 2) {
+      m0 = max3(m0, s[0][r], s[0][r + 1]);
+      m1 = max3(m1, s[1][r], s[1][r + 1]);
+    }
+    return pair_max(max3(m0, m1, fmaxf(s[0][15], s[1][15])));
   };
-  // Whether any reference of the wave has to move (wave-uniform).  Looks at the lanes' partial maxima only: a row
-  // maximum above the threshold shows in one of its four lanes, and a row maximum below minus the threshold
-  // shows in all four, so "some lane below" can only fire early, never late -- the move itself works with the
-  // true row maxima and is harmless when it was not strictly needed.
-  auto ref_must_move = [&](const float (&mx)[2], int blk) -> bool {
-    const float hi = fmaxf(mx[0], mx[1]), lo = fminf(mx[0], mx[1]);
-    const bool move = hi > kRescaleThreshold || (blk == kb_begin && lo < -kRescaleThreshold);
+  auto ref_must_move = [&](float mx, int blk) -> bool {  // wave-uniform
+    const bool move = mx > kRescaleThreshold || (blk == kb_begin && mx < -kRescaleThreshold);
     return __builtin_amdgcn_ballot_w64(move) != 0;
   };
-  auto ref_move = [&](f32x4 (&s)[4][2], const float (&part)[2], int blk, float (&alpha)[2]) {
+  auto ref_move = [&](f32x16 (&s)[2], float mx, int blk) -> float {
     any_ref = true;
+    const float d = blk == kb_begin ? mx : fmaxf(mx, 0.f);
+    const float alpha = blk == kb_begin ? 1.0f : __builtin_amdgcn_exp2f(-d);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const float mxt = quad_max(part[t]);  // the row maximum: over the four lanes that share the query
-      const float d = blk == kb_begin ? mxt : fmaxf(mxt, 0.f);
-      alpha[t] = blk == kb_begin ? 1.0f : __builtin_amdgcn_exp2f(-d);
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+      for (int r = 0; r < 16; ++r) s[kt][r] -= d;
+    m_ref += d;
+    l_run *= alpha;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) s[kt][t][e] -= d;
-      m_ref[t] += d;
-      l_run[t] *= alpha[t];
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int dt = 0; dt < 8; ++dt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) oacc[dt][t][e] *= alpha[t];
-    }
+      for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+    return alpha;
   };
-  // Entry n (0..31) of P = exp2(S'), in the order the second product consumes them: 32-key chunk n / 16, query
-  // column (n / 8) % 2, word (n / 2) % 4 of that column's B operand -- words 0, 1 hold keys 4q .. 4q + 3 of the
-  // chunk's first key tile, words 2, 3 those of its second -- low or high half n % 2.  The row sum adds the fp32
-  // values with plain v_add_f32 (v_dot2c_f32_bf16 on the packed pair would be one instruction, but it executes
-  // on the matrix pipe and was measured to cost a third of the MFMA rate).
+  // entry e (0..31) of P = exp2(S'): score s[e/16][e%16]; two entries pack into one bf16x2 word of the PV
+  // operand.  The row sum adds the fp32 values with plain v_add_f32 (v_dot2c_f32_bf16 on the packed pair
+  // would be one instruction, but it executes on the matrix pipe and was measured to cost a third of the
+  // MFMA rate).
   // Each result is pinned where it is computed by an empty volatile asm that "uses" it: the exponential, the
   // convert and the add are pure, and the optimiser otherwise sinks them to the block of their first use (the
   // PV MFMAs behind the next branch, the row sum at the end of the interval), past the scheduling barriers:
   // the MFMA slots they were written into then run bare and the VALU work runs in MFMA-free clumps.
-  float p_even = 0.f, lsum[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
-  auto exp_entry = [&](const f32x4 (&s)[4][2], uint32_t (&pw)[2][2][4], int n) {
-    const int ch = n >> 4, t = (n >> 3) & 1, w = (n >> 1) & 3;
-    float pv = __builtin_amdgcn_exp2f(s[2 * ch + (w >> 1)][t][2 * (w & 1) + (n & 1)]);
-    if (n & 1) {
-      uint32_t word = pack_bf16x2(p_even, pv);
-      lsum[t][1] += pv;
-      asm volatile("" : "+v"(word), "+v"(lsum[t][1]));
-      pw[ch][t][w] = word;
+  float p_even = 0.f, lsum0 = 0.f, lsum1 = 0.f;
+  auto exp_entry = [&](const f32x16 (&s)[2], uint32_t (&pw)[2][8], int e) {
+    float pv = __builtin_amdgcn_exp2f(s[e >> 4][e & 15]);
+    if (e & 1) {
+      uint32_t w = pack_bf16x2(p_even, pv);
+      lsum1 += pv;
+      asm volatile("" : "+v"(w), "+v"(lsum1));
+      pw[e >> 4][(e & 15) >> 1] = w;
     } else {
-      lsum[t][0] += pv;
-      asm volatile("" : "+v"(pv), "+v"(lsum[t][0]));
+      lsum0 += pv;
+      asm volatile("" : "+v"(pv), "+v"(lsum0));
       p_even = pv;
     }
   };
-  // first block: S(0) with nothing to overlap
-  auto qk = [&](f32x4 (&s)[4][2], int stage) {
+  auto qk = [&](f32x16 (&s)[2], int stage) {
     const uint8_t* sK = smem + stage * kTile;
 #pragma unroll
-    for (int dc = 0; dc < 4; ++dc)
+    for (int kc = 0; kc < 8; ++kc) {
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + lane_k[dc] + kt * 4096);
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-          s[kt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[t][dc], dc == 0 ? zero4 : s[kt][t], 0, 0, 0);
+      for (int kt = 0; kt < 2; ++kt) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + lane_k[kc] + kt * 8192);
+        s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kc], kc == 0 ? zero16 : s[kt], 0, 0, 0);
       }
+    }
   };
   typedef short v8i16 __attribute__((ext_vector_type(8)));
   // one interval; `stage` (= kb % 4) is a literal so that every LDS offset folds into an immediate.
   // pw_cur holds entries 0..kExpEarly-1 of P(kb) on entry; pw_next holds those of P(kb+1) on exit.
-  auto interval = [&](int kb, int stage, f32x4 (&s_cur)[4][2], f32x4 (&s_next)[4][2], uint32_t (&pw_cur)[2][2][4],
-                      uint32_t (&pw_next)[2][2][4]) {
+  auto interval = [&](int kb, int stage, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], uint32_t (&pw_cur)[2][8],
+                      uint32_t (&pw_next)[2][8]) {
     interval_head(kb);
     // The next block's four 1 KiB pieces go out between the MFMAs, K in stage 1 and V in stage 2: the CU's
     // one address path takes ~25 cycles per piece, and a wave whose load queues behind the other waves'
     // loads cannot issue its MFMAs meanwhile (32 pieces at once right after the barrier cost every wave
     // 500-800 cycles).
-    constexpr int kLoadSlots[4] = {3, 11, 7, 13};  // in operand fragments (= MFMA pairs)
-    // ---- stage 1: 16 operand fragments, each = [LDS read of the K fragment two fragments ahead, two MFMAs of
-    //      S(kb+1) (the two query columns), entries of P(kb)]; sched_barrier pins the order
+    constexpr int kLoadSlots[4] = {3, 11, 7, 13};
+    // ---- stage 1: 16 slots, each = [LDS read of the K fragment two MFMAs ahead, one MFMA of S(kb+1),
+    //      one or two entries of P(kb)]; sched_barrier pins the order
     const uint8_t* sK = smem + ((stage + 1) % kStages) * kTile;
-    auto k_frag = [&](int f) {  // fragment f of the block: d chunk f/4, key tile f%4
-      return *reinterpret_cast<const bf16x8*>(sK + lane_k[f >> 2] + (f & 3) * 4096);
+    auto k_frag = [&](int i) {  // MFMA i of the block: k-chunk i/2, key tile i%2
+      return *reinterpret_cast<const bf16x8*>(sK + lane_k[i >> 1] + (i & 1) * 8192);
     };
     const uint8_t* sV = smem + stage * kTile;  // lane_v carries the offset of the V region
-    auto v_frag = [&](int f) {  // fragment f: 32-key chunk f/8, d tile f%8; keys 4q .. 4q + 3 of both 16-key halves
-      const uint8_t* src = sV + lane_v[f & 7] + (f >> 3) * 32 * 256;
+    auto v_frag = [&](int j) {  // MFMA j: 16-key chunk j/4 (kt = j/8, ch = (j/4)%2), d tile j%4
+      const uint8_t* src = sV + lane_v[j & 3] + (j >> 2) * 16 * 256;
       const v4i16 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)src);
       const v4i16 hi =
-          __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(src + 16 * 256));
+          __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(src + 8 * 256));
       const v8i16 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       return __builtin_bit_cast(bf16x8, both);
     };
-    // operand fragments are read kAhead fragments before their use; the last slots of stage 1 already fetch
+    // operand fragments are read kAhead MFMAs before their use; the last slots of stage 1 already fetch
     // the first V^T fragments of stage 2 (block kb landed long ago), so only stage 1 starts cold
+    constexpr int kLate = 32 - kExpEarly;  // entries left for stage 1; the first kLate-16 slots take two
     bf16x8 kf[kAhead + 1], vf[kAhead + 1];
 #pragma unroll
-    for (int f = 0; f < kAhead; ++f) kf[f] = k_frag(f);
-    int n = kExpEarly;
+    for (int i = 0; i < kAhead; ++i) kf[i] = k_frag(i);
+    int e = kExpEarly;
 #pragma unroll
-    for (int f = 0; f < 16; ++f) {
-      if (f + kAhead < 16)
-        kf[(f + kAhead) % (kAhead + 1)] = k_frag(f + kAhead);
+    for (int i = 0; i < 16; ++i) {
+      if (i + kAhead < 16)
+        kf[(i + kAhead) % (kAhead + 1)] = k_frag(i + kAhead);
       else
-        vf[(f + kAhead - 16) % (kAhead + 1)] = v_frag(f + kAhead - 16);
-      const int dc = f >> 2, kt = f & 3;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        s_next[kt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[f % (kAhead + 1)], qf[t][dc],
-                                                                dc == 0 ? zero4 : s_next[kt][t], 0, 0, 0);
-        // 32 - kExpEarly entries over 32 slots: one per slot until they are done
-        if (n < 32) exp_entry(s_cur, pw_cur, n++);
-        if (t == 0 && f == kLoadSlots[0]) issue_piece((stage + 3) % kStages, 0);
-        if (t == 0 && f == kLoadSlots[1]) issue_piece((stage + 3) % kStages, 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+        vf[(i + kAhead - 16) % (kAhead + 1)] = v_frag(i + kAhead - 16);
+      const int kt = i & 1;
+      s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % (kAhead + 1)], qf[i >> 1], i < 2 ? zero16 : s_next[kt], 0, 0, 0);
+      exp_entry(s_cur, pw_cur, e++);
+      if (i < kLate - 16) exp_entry(s_cur, pw_cur, e++);
+      if (i == kLoadSlots[0]) issue_piece((stage + 3) % kStages, 0);
+      if (i == kLoadSlots[1]) issue_piece((stage + 3) % kStages, 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      l_run[t] += lsum[t][0] + lsum[t][1];
-      lsum[t][0] = lsum[t][1] = 0.f;
-    }
-    // ---- stage 2: O^T += V^T P^T, 16 operand fragments = [transposing LDS reads of a V^T operand, two MFMAs]
-    auto pv_frag = [&](int f, int t) {
-      if (t == 0 && f + kAhead < 16) vf[(f + kAhead) % (kAhead + 1)] = v_frag(f + kAhead);
-      const int ch = f >> 3, dt = f & 7;
-      const u32x4 w = {pw_cur[ch][t][0], pw_cur[ch][t][1], pw_cur[ch][t][2], pw_cur[ch][t][3]};
-      oacc[dt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[f % (kAhead + 1)], __builtin_bit_cast(bf16x8, w),
-                                                            oacc[dt][t], 0, 0, 0);
+    l_run += lsum0 + lsum1;
+    lsum0 = lsum1 = 0.f;
+    // ---- stage 2: O^T += V^T P^T, 16 slots = [transposing LDS reads of a V^T operand, one MFMA].
+    //      16-key chunk (kt, ch): slots 8g..8g+7 = keys {4g..4g+3, 8+4g..8+4g+3}
+    auto pv_slot = [&](int j) {
+      if (j + kAhead < 16) vf[(j + kAhead) % (kAhead + 1)] = v_frag(j + kAhead);
+      const int kt = j >> 3, ch = (j >> 2) & 1, dt = j & 3;
+      const u32x4 w = {pw_cur[kt][4 * ch + 0], pw_cur[kt][4 * ch + 1], pw_cur[kt][4 * ch + 2], pw_cur[kt][4 * ch + 3]};
+      oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[j % (kAhead + 1)], __builtin_bit_cast(bf16x8, w), oacc[dt], 0, 0, 0);
     };
-    constexpr int kScanFrags = 4;  // PV fragments issued before the block maximum of S(kb+1) is looked at
+    constexpr int kScanSlots = 4;  // PV MFMAs issued before the block maximum of S(kb+1) is looked at
 #pragma unroll
-    for (int f = 0; f < kScanFrags; ++f)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        pv_frag(f, t);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    for (int j = 0; j < kScanSlots; ++j) {
+      pv_slot(j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     if (__builtin_expect(kb + 1 < kb_end, 1)) {
       mask_tail(s_next, kb + 1);
-      float mx[2] = {0.f, 0.f};
-      if (SCAN) ref_scan(s_next, mx);
+      const float mx = SCAN ? ref_scan(s_next, kb + 1) : 0.f;
       if (SCAN && __builtin_expect(ref_must_move(mx, kb + 1), 0)) {
         // rare: O, l and the scores of block kb+1 move to the new reference now; the part of P(kb) that
         // the remaining PV MFMAs still have to accumulate follows (one more bf16 rounding on it)
-        float alpha[2];
-        ref_move(s_next, mx, kb + 1, alpha);
+        const float alpha = ref_move(s_next, mx, kb + 1);
 #pragma unroll
-        for (int ch = 0; ch < 2; ++ch)
+        for (int j = kScanSlots; j < 16; j += 4)
 #pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-              uint32_t& word = pw_cur[ch][t][w];
-              word = pack_bf16x2(bf16_lo(word) * alpha[t], bf16_hi(word) * alpha[t]);
-            }
+          for (int w = 0; w < 4; ++w) {
+            uint32_t& word = pw_cur[j >> 3][4 * ((j >> 2) & 1) + w];
+            word = pack_bf16x2(bf16_lo(word) * alpha, bf16_hi(word) * alpha);
+          }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
     // (in the last interval the entries below come from a block that does not exist and are dropped)
-    int n2 = 0;
+    int e2 = 0;
 #pragma unroll
-    for (int f = kScanFrags; f < 16; ++f)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        pv_frag(f, t);
-        // kExpEarly entries over the 2 (16 - kScanFrags) remaining slots: every second slot
-        if (t == 0 && n2 < kExpEarly) exp_entry(s_next, pw_next, n2++);
-        if (t == 1 && f == kLoadSlots[2]) issue_piece((stage + 3) % kStages, 2);
-        if (t == 1 && f == kLoadSlots[3]) issue_piece((stage + 3) % kStages, 3);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+    for (int j = kScanSlots; j < 16; ++j) {
+      pv_slot(j);
+      // kExpEarly entries over the 16 - kScanSlots remaining slots, the surplus in the first ones
+      exp_entry(s_next, pw_next, e2++);
+      if (j - kScanSlots < kExpEarly - (16 - kScanSlots)) exp_entry(s_next, pw_next, e2++);
+      if (j == kLoadSlots[2]) issue_piece((stage + 3) % kStages, 2);
+      if (j == kLoadSlots[3]) issue_piece((stage + 3) % kStages, 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
-  f32x4 sA[4][2], sB[4][2];
-  uint32_t pwA[2][2][4], pwB[2][2][4];
+  f32x16 sA[2], sB[2];
+  uint32_t pwA[2][8], pwB[2][8];
   __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): block 0 has landed
   __builtin_amdgcn_s_barrier();
   qk(sA, 0);
   {
     mask_tail(sA, kb_begin);
     if (SCAN) {
-      float mx[2], alpha[2];
-      ref_scan(sA, mx);
-      if (ref_must_move(mx, kb_begin)) ref_move(sA, mx, kb_begin, alpha);
+      const float mx = ref_scan(sA, kb_begin);
+      if (ref_must_move(mx, kb_begin)) ref_move(sA, mx, kb_begin);
     }
 #pragma unroll
-    for (int n = 0; n < kExpEarly; ++n) exp_entry(sA, pwA, n);
+    for (int e = 0; e < kExpEarly; ++e) exp_entry(sA, pwA, e);
   }
   for (int kb = kb_begin; kb < kb_end; kb += 4) {  // stage of block kb = (kb - kb_begin) % 4
     interval(kb, 0, sA, sB, pwA, pwB);
@@ -558,32 +519,26 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
   }
   __builtin_amdgcn_s_waitcnt(0);  // drain trailing async loads
 
-  // ---- lane (q, i): queries 16t + i, d = 16dt + 4q + e
-  float l_row[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) l_row[t] = quad_sum(l_run[t]);
+  // ---- lane (g, j): query j, d = dt*32 + 8*(r/4) + 4g + r%4
+  const float l_row = pair_sum(l_run);
+  const int64_t row = q0 + li;
   if (!SPLIT || (kb_begin == 0 && kb_end == nkb)) {  // the whole key axis: normalise and store
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int64_t row = q0 + t * 16 + i16;
-      if (row < Sq) store_output(p, b, h, row, q4, oacc, t, 1.0f / l_row[t]);
-    }
+    if (row < Sq) store_output(p, b, h, row, g, oacc, 1.0f / l_row);
   } else {                               // a part: leave O, l and the reference for the merge
-    const int tu = unit - sp.full_units;
-    const int first_piece = (tu * nkb) / sp.len;
-    const int my_piece = (tu * nkb + kb_begin) / sp.len;
-    float* slot = sp.slots + (int64_t)(tu * sp.max_parts + (my_piece - first_piece)) * kSlotFloats;
+    const int t = unit - sp.full_units;
+    const int first_piece = (t * nkb) / sp.len;
+    const int my_piece = (t * nkb + kb_begin) / sp.len;
+    float* slot = sp.slots + (int64_t)(t * sp.max_parts + (my_piece - first_piece)) * kSlotFloats;
 #pragma unroll
-    for (int dt = 0; dt < 8; ++dt)
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-        *reinterpret_cast<f32x4*>(slot + (((dt * 2 + t) * 8 + wave) * 64 + lane) * 4) = oacc[dt][t];
-    if (q4 == 0) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        slot[kSlotOFloats + wave * 32 + t * 16 + i16] = l_row[t];
-        slot[kSlotOFloats + QB + wave * 32 + t * 16 + i16] = m_ref[t];
+      for (int rq = 0; rq < 4; ++rq) {
+        const f32x4 v = {oacc[dt][4 * rq + 0], oacc[dt][4 * rq + 1], oacc[dt][4 * rq + 2], oacc[dt][4 * rq + 3]};
+        *reinterpret_cast<f32x4*>(slot + ((((dt * 4 + rq) * 8 + wave) * 2 + g) * 32 + li) * 4) = v;
       }
+    if (g == 0) {
+      slot[kSlotOFloats + wave * 32 + li] = l_row;
+      slot[kSlotOFloats + QB + wave * 32 + li] = m_ref;
     }
   }
   }  // parts
@@ -591,25 +546,25 @@ __global__ __launch_bounds__(512) void attn_plain_kernel(dsx_attn_params p, Attn
 
 // Combines the parts of every split unit: O = sum_i O_i 2^(m_i - m), l likewise, m = max_i m_i.
 // Same lane <-> (query, d) mapping as the attention kernel, so the slots are read as they were written.
-// blockIdx.y picks one of the sixteen (dt, t) groups of four output columns: a unit's merge is spread over
+// blockIdx.y picks one of the sixteen (dt, rq) groups of four output columns: a unit's merge is spread over
 // sixteen workgroups, each reading one 16-byte vector per lane and part (a unit cut into many parts would
 // otherwise be read, 128 KiB per part, by a single workgroup).
 __global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, AttnSplit sp) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int q4 = lane >> 4, i16 = lane & 15;
+  const int g = lane >> 5, li = lane & 31;
   const int nqb = (int)((p.sq[0] + p.sq[1] + QB - 1) / QB);
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int nkb = (int)((p.skv[0] + p.skv[1] + KB - 1) / KB);
-  const int tu = blockIdx.x;
-  const int dt = (int)blockIdx.y >> 1, t = (int)blockIdx.y & 1;
-  const int first_piece = (tu * nkb) / sp.len, last_piece = ((tu + 1) * nkb - 1) / sp.len;
+  const int t = blockIdx.x;
+  const int dt = (int)blockIdx.y >> 2, rq = (int)blockIdx.y & 3;
+  const int first_piece = (t * nkb) / sp.len, last_piece = ((t + 1) * nkb - 1) / sp.len;
   const int np = last_piece - first_piece + 1;
   if (np == 1) return;  // the unit was covered by one piece, which wrote the output itself
-  const int unit = sp.full_units + tu;
+  const int unit = sp.full_units + t;
   const int qblk = unit % nqb;
   const int h = (unit / nqb) % p.heads, b = unit / (nqb * p.heads);
-  const float* base = sp.slots + (int64_t)tu * sp.max_parts * kSlotFloats;
-  const int qi = wave * 32 + t * 16 + i16;
+  const float* base = sp.slots + (int64_t)t * sp.max_parts * kSlotFloats;
+  const int qi = wave * 32 + li;
   float m = -INFINITY;
   for (int i = 0; i < np; ++i) m = fmaxf(m, base[(int64_t)i * kSlotFloats + kSlotOFloats + QB + qi]);
   f32x4 o = {0.f, 0.f, 0.f, 0.f};
@@ -618,7 +573,7 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, Attn
     const float* slot = base + (int64_t)i * kSlotFloats;
     const float w = __builtin_amdgcn_exp2f(slot[kSlotOFloats + QB + qi] - m);
     l += slot[kSlotOFloats + qi] * w;
-    const f32x4 v = *reinterpret_cast<const f32x4*>(slot + (((dt * 2 + t) * 8 + wave) * 64 + lane) * 4);
+    const f32x4 v = *reinterpret_cast<const f32x4*>(slot + ((((dt * 4 + rq) * 8 + wave) * 2 + g) * 32 + li) * 4);
 #pragma unroll
     for (int c = 0; c < 4; ++c) o[c] += v[c] * w;
   }
@@ -631,7 +586,7 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(dsx_attn_params p, Attn
   u32x2 w2;
   w2.x = pack_bf16x2(o[0] * inv, o[1] * inv);
   w2.y = pack_bf16x2(o[2] * inv, o[3] * inv);
-  *reinterpret_cast<u32x2*>(dst + dt * 16 + 4 * q4) = w2;
+  *reinterpret_cast<u32x2*>(dst + dt * 32 + 8 * rq + 4 * g) = w2;
 }
 
 }  // namespace
@@ -708,8 +663,13 @@ int launch_attn_plain(const dsx_attn_params& p, void* scratch, int64_t scratch_b
   const int64_t Sq = p.sq[0] + p.sq[1];
   const int64_t units = ((Sq + QB - 1) / QB) * p.heads * p.batch;
   if (units > (1ll << 30)) return DSX_EBADSHAPE;
+  // Three full rounds of workgroups and more run into the chip's power limit, where the 16x16x32 form of the kernel
+  // is the faster one (attn_plain16.hip); below that this one is.
+  const int cus = device_cus();
+  const bool qpre_any = p.rope || p.q_norm_w[0] || p.q_norm_w[1];
+  if (cus > 0 && units >= 3 * (int64_t)cus && !qpre_any) return launch_attn_plain16(p, units, st);
   AttnSplit sp;
-  const int64_t need = plan_split(p, device_cus(), sp);
+  const int64_t need = plan_split(p, cus, sp);
   if (need == 0 || !scratch || scratch_bytes < need || ((uintptr_t)scratch & 15))
     sp = AttnSplit{(int)units, 0, 0, 1, 1, nullptr, 0};
   else

@@ -313,3 +313,45 @@ def test_device_side_score_bound_not_with_fused_preprocessing(dev):
         ops.attention_bhsd(q, k, v, q_norm_w=w, qk_norm2_max=torch.ones(2, device=dev))
     with pytest.raises(ValueError):
         ops.attention_bhsd(q, k, v, qk_norm2_max=torch.ones(3, device=dev))
+
+
+@pytest.mark.parametrize("variant", ["scan", "score_bound", "device_bound", "far_reference", "two_segments"])
+def test_many_round_launches_take_the_16x16_form_and_agree(dev, variant):
+    """Launches of three full rounds of workgroups and more (>= 768 units of 256 queries on 256 compute units) run
+    on the 16x16x32 form of the kernel (attn_plain16.hip); fewer units run on the 32x32x16 form.  Same operation:
+    the rows of a many-round call agree with torch's fp32 SDPA on the device to the bar, and with the same heads
+    computed in a small launch (the other form) to a few bf16 roundings.  Ragged query and key counts; the running
+    maximum, a caller's score bound, the device-side bound, a softmax reference that has to move (scores far from
+    zero), and the two-segment (joint) form each take their own path through the kernel."""
+    from diffsynth_engine_amd import ops
+
+    B, H, Sq, Skv = 2, 24, 4200, 1111  # 17 query blocks x 24 heads x 2 = 816 units; 1111 = 17 x 64 + 23 keys
+    g = torch.Generator(device=dev).manual_seed(5)
+    q, k, v = [torch.randn(B, H, n, 128, generator=g, device=dev).bfloat16() for n in (Sq, Skv, Skv)]
+    kw = {}
+    if variant == "far_reference":
+        q = q * 12  # log2-domain scores of std ~17: block maxima beyond 64 move the softmax reference
+    elif variant != "scan":
+        q = torch.nn.functional.normalize(q.float(), dim=-1).mul(11.3).bfloat16()
+        k = torch.nn.functional.normalize(k.float(), dim=-1).mul(11.3).bfloat16()
+        if variant == "score_bound":
+            kw["score_bound"] = 11.6
+        elif variant == "device_bound":
+            n2 = lambda t: t.float().square().sum(-1).max()
+            kw["qk_norm2_max"] = torch.stack([n2(q), n2(k)])
+    if variant == "two_segments":
+        out = ops.attention_bhsd(q[:, :, :500], k[:, :, :300], v[:, :, :300], q2=q[:, :, 500:], k2=k[:, :, 300:],
+                                 v2=v[:, :, 300:])
+        got = torch.cat(out, dim=2)
+    else:
+        got = ops.attention_bhsd(q, k, v, **kw)
+    heads = (0, 13, 23)
+    want = torch.nn.functional.scaled_dot_product_attention(q[:, heads, :].float(), k[:, heads, :].float(),
+                                                            v[:, heads, :].float())
+    # (q is multiplied by scale * log2(e) once and the product rounded to bf16, so a score s carries an absolute error
+    # of about |s| * 2^-9 in the exponent: far inside the bar for scores of a few units, and the x12 case, whose rows
+    # are nearly one-hot, is held to 3 x the bar, as in test_key_range_split_of_the_last_round)
+    assert _rel_err(got[:, heads, :], want) <= (3 * TOL if variant == "far_reference" else TOL)
+    small = ops.attention_bhsd(q[:1, :2].contiguous(), k[:1, :2].contiguous(), v[:1, :2].contiguous(),
+                               **{n: t for n, t in kw.items() if n == "score_bound"})  # 34 units: the other form
+    assert _rel_err(got[:1, :2], small) <= 1e-2
