@@ -747,6 +747,27 @@ def main():
                 del gstep
             other["%dx%d" % (side * 8, side * 8)] = entry
         result["detail"]["flux_other_image_sizes"] = other
+        # the same step with an unfused rank-16 LoRA on every one of the 228 block linears (LoRALinear.forward,
+        # models/basic/lora.py:137-141): the updates ride the main products as 128 more columns of their reduction
+        # axis, one small down-projection launch per linear
+        names = [n for n in runner.lin if n.startswith(("blocks.", "single_blocks."))]
+        for n in names:
+            L = runner.lin[n]
+            L.add_lora((torch.randn(16, L.k, generator=g, device=dev) * 0.01).to(torch.bfloat16),
+                       (torch.randn(L.n, 16, generator=g, device=dev) * 0.01).to(torch.bfloat16), 1.0)
+        riding = sum(runner.lin[n]._extension() is not None for n in names)
+        for _ in range(2):
+            out_l = runner(**inp)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            out_l = runner(**inp)
+        torch.cuda.synchronize()
+        ms_l = (time.perf_counter() - t0) * 1e3 / 5
+        assert torch.isfinite(out_l.float()).all().item(), "non-finite output"
+        result["detail"]["lora_rank16_on_all_block_linears"] = {
+            "linears": len(names), "riding_the_main_product": riding, "ms_per_step": round(ms_l, 2),
+            "overhead_frac": round(ms_l / ms - 1.0, 4)}
     del runner
     torch.cuda.empty_cache()
     if not args.no_micro:

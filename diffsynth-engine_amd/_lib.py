@@ -21,7 +21,7 @@ DSX_EARCH = -3
 DSX_ELAUNCH = -4
 DSX_ENULL = -5
 DSX_EWORKSPACE = -6
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class AttnParams(ctypes.Structure):
@@ -71,6 +71,9 @@ class GemmProblem(ctypes.Structure):
         ("rope", c_void_p), ("rope_sb", c_int64), ("rope_pos0", c_int64), ("rope_rows", c_int64),
         ("norm_eps", c_float),
         ("qk_heads", ctypes.c_int32),
+        ("a_ext", c_void_p), ("lda_ext", c_int64),
+        ("w_ext", c_void_p), ("ldw_ext", c_int64),
+        ("K_ext", c_int64),
     ]
 
 
@@ -90,6 +93,8 @@ SIGNATURES = {
                                             c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
                                             c_int64, c_int64, c_int64, c_void_p]),
     "dsx_fp8_gemm_grouped": (c_int, [ctypes.POINTER(GemmProblem), c_int, c_void_p]),
+    "dsx_lora_down": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                              c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "dsx_fp8_gemv_rowscale": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "dsx_concat_gelu_tanh": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,

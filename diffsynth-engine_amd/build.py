@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libdsx.so")
-SOURCES = ["capi.hip", "quant.hip", "fp8_gemm.hip", "attn_fwd.hip", "attn_plain.hip", "attn_plain16.hip", "epilogue.hip"]
+SOURCES = ["capi.hip", "quant.hip", "fp8_gemm.hip", "attn_fwd.hip", "attn_plain.hip", "attn_plain16.hip", "epilogue.hip", "lora.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 HIPCC_FLAGS = [

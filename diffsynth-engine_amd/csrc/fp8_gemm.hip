@@ -61,6 +61,11 @@ struct GemmArgs {
   int64_t rope_sb;        // per batch entry m / rows_per_batch
   int rope_pos0, qk_heads;
   float qk_eps;
+  // optional second segment of the reduction axis (main kernel only): K2 more columns from (a2, w2)
+  const uint8_t* a2;
+  const uint8_t* w2;
+  int64_t lda2, ldw2;
+  int K2;
 };
 
 // Two problems in one grid: logical tiles [0, tiles of p[0]) belong to p[0], the rest to p[1].
@@ -80,7 +85,7 @@ __device__ __forceinline__ GemmArgs pick(const GemmPair& q, bool second) {
   DSX_PICK(tiles_m); DSX_PICK(tiles_n); DSX_PICK(resid); DSX_PICK(gate); DSX_PICK(ldr); DSX_PICK(gate_sb);
   DSX_PICK(rows_per_batch); DSX_PICK(w_row_scale);
   DSX_PICK(qk_wq); DSX_PICK(qk_wk); DSX_PICK(rope); DSX_PICK(rope_sb); DSX_PICK(rope_pos0); DSX_PICK(qk_heads);
-  DSX_PICK(qk_eps);
+  DSX_PICK(qk_eps); DSX_PICK(a2); DSX_PICK(w2); DSX_PICK(lda2); DSX_PICK(ldw2); DSX_PICK(K2);
 #undef DSX_PICK
   return r;
 }
@@ -373,7 +378,9 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 // (WM 2, MT 8 -- four waves of 128 x 128 on a 256 x 256 tile, accumulators in 256 AccVGPRs -- compiles and passes
 // the same tests; it is not instantiated, see above.)
 // Same K order in every form, so a row's bits do not depend on which of them computed it.
-template <bool RESID, bool QK, int WM = 4, int MT = 4>
+// EXT: a second segment of the reduction axis may follow the first (GemmArgs::K2); a variant of its own, because the
+// cross-over's bookkeeping costs the plain loop 3 %.
+template <bool RESID, bool QK, int WM = 4, int MT = 4, bool EXT = false>
 __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
   constexpr int PW = 16 / WM;  // 1 KiB pieces of a W unit (256 rows) per wave
   constexpr int PA = MT;       // 1 KiB pieces of an A unit (32 WM MT rows) per wave
@@ -415,7 +422,29 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
   }
   const uint8_t* w_base = p.w + (int64_t)n0 * p.ldw;
   const uint8_t* a_base = p.a + (int64_t)m0 * p.lda;
-  const int nu = p.K / UK;
+  // Units [0, nu1) come from (a, w), units [nu1, nu) from the optional second segment (a2, w2), whose rows are the
+  // same rows at other leading dimensions: the per-lane offsets are re-formed once, when the loads cross over.
+  const int nu1 = p.K / UK;
+  const int nu = EXT ? nu1 + p.K2 / UK : nu1;
+  const uint8_t* w2_base = p.w2 + (int64_t)n0 * p.ldw2 - (int64_t)nu1 * UK;  // so that unit j sits at base + j * UK
+  const uint8_t* a2_base = p.a2 + (int64_t)m0 * p.lda2 - (int64_t)nu1 * UK;
+  auto cross_over = [&](int op) {
+    if (op == 0) {
+#pragma unroll
+      for (int i = 0; i < PW; ++i) {
+        const int row = (wave * PW + i) * 8 + ld_r;
+        const int c = ld_p ^ ((row >> 1) & 7);
+        w_off[i] = (uint32_t)(min(n0 + row, p.N - 1) - n0) * (uint32_t)p.ldw2 + c * 16;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < PA; ++i) {
+        const int row = (wave * PA + i) * 8 + ld_r;
+        const int c = ld_p ^ ((row >> 1) & 7);
+        a_off[i] = (uint32_t)(min(m0 + row, p.M - 1) - m0) * (uint32_t)p.lda2 + c * 16;
+      }
+    }
+  };
   // The async loads are issued as assembly in the scalar-base + 32-bit-lane-offset form: the builtin takes a
   // 64-bit per-lane address, and eight of those (plus their increments) are sixteen registers the eight-wave
   // form, at 256 per wave, does not have.  M0 carries the LDS destination; nothing else here uses M0.
@@ -426,8 +455,9 @@ __global__ __launch_bounds__(128 * WM) void fp8_gemm_kernel(GemmPair q) {
   auto issue_load = [&](int j, int op, int i) {
     const int slot = (2 * j + op) % NSLOT;
     j = min(j, nu - 1);
+    if (EXT && i == 0 && j == nu1 && p.K2 > 0) cross_over(op);  // (pieces of a unit go out in order, units in order)
     const uint32_t dst = lds0 + slot * kUnitBytes + (wave_u * (op ? PA : PW) + i) * 1024;
-    const uint8_t* ub = (op ? a_base : w_base) + (int64_t)j * UK;
+    const uint8_t* ub = (EXT && j >= nu1 ? (op ? a2_base : w2_base) : (op ? a_base : w_base)) + (int64_t)j * UK;
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(op ? a_off[i] : w_off[i]), "s"(ub), "s"(dst)
@@ -783,9 +813,12 @@ static int gemm_set_attributes() {
   static PerDeviceOnce once;
   return per_device_once(once, [](int) {
     const void* kernels[] = {
-        (const void*)fp8_gemm_kernel<false, false, 4, 4>, (const void*)fp8_gemm_kernel<true, false, 4, 4>,
-        (const void*)fp8_gemm_kernel<false, true, 4, 4>,  (const void*)fp8_gemm_kernel<false, false, 2, 4>,
-        (const void*)fp8_gemm_kernel<true, false, 2, 4>,  (const void*)fp8_gemm_kernel<false, true, 2, 4>};
+        (const void*)fp8_gemm_kernel<false, false, 4, 4>,       (const void*)fp8_gemm_kernel<true, false, 4, 4>,
+        (const void*)fp8_gemm_kernel<false, true, 4, 4>,        (const void*)fp8_gemm_kernel<false, false, 2, 4>,
+        (const void*)fp8_gemm_kernel<true, false, 2, 4>,        (const void*)fp8_gemm_kernel<false, true, 2, 4>,
+        (const void*)fp8_gemm_kernel<false, false, 4, 4, true>, (const void*)fp8_gemm_kernel<true, false, 4, 4, true>,
+        (const void*)fp8_gemm_kernel<false, true, 4, 4, true>,  (const void*)fp8_gemm_kernel<false, false, 2, 4, true>,
+        (const void*)fp8_gemm_kernel<true, false, 2, 4, true>,  (const void*)fp8_gemm_kernel<false, true, 2, 4, true>};
     for (const void* k : kernels)
       if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kMainLdsBytes) != hipSuccess)
         return (int)DSX_ELAUNCH;
@@ -810,6 +843,28 @@ static bool gemm_main_kernel_ok(dsx::GemmArgs& p) {
 
 constexpr int kHalfTileThreshold = 128;
 
+// The instantiation for one launch: epilogue kind of the first problem (pairs agree on it), waves along m, and
+// whether either problem continues its reduction axis in a second segment.
+template <int WM>
+static void launch_form(const dsx::GemmPair& q, const dsx::GemmArgs& p0, bool ext, int grid, hipStream_t st) {
+  using namespace dsx;
+  const dim3 g((unsigned)grid), b(128 * WM);
+#define DSX_GO(R, Q)                                                                   \
+  do {                                                                                 \
+    if (ext)                                                                           \
+      fp8_gemm_kernel<R, Q, WM, 4, true><<<g, b, kMainLdsBytes, st>>>(q);              \
+    else                                                                               \
+      fp8_gemm_kernel<R, Q, WM, 4, false><<<g, b, kMainLdsBytes, st>>>(q);             \
+  } while (0)
+  if (p0.resid)
+    DSX_GO(true, false);
+  else if (p0.qk_heads > 0)
+    DSX_GO(false, true);
+  else
+    DSX_GO(false, false);
+#undef DSX_GO
+}
+
 // One launch of the main kernel over one or two problems (of the same kind: plain, residual or qk epilogue).
 static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStream_t st) {
   using namespace dsx;
@@ -818,6 +873,7 @@ static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStre
   q.p[1] = p1 ? *p1 : p0;
   q.total0 = p0.tiles_m * p0.tiles_n;
   q.total = q.total0 + (p1 ? p1->tiles_m * p1->tiles_n : 0);
+  const bool ext = p0.K2 > 0 || (p1 && p1->K2 > 0);
   // At most half the compute units' worth of 256 x 256 tiles (MI355X: 256): tiles of 128 token rows fill twice
   // as many, and the four-wave form of the kernel runs them (same wave tile and K order: same bits).
   if (q.total <= kHalfTileThreshold) {
@@ -826,21 +882,11 @@ static int launch_main(const dsx::GemmArgs& p0, const dsx::GemmArgs* p1, hipStre
     q.total0 = q.p[0].tiles_m * p0.tiles_n;
     q.total = q.total0 + (p1 ? q.p[1].tiles_m * p1->tiles_n : 0);
     const int grid = ((q.total + 7) / 8) * 8;
-    if (p0.resid)
-      fp8_gemm_kernel<true, false, 2, 4><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
-    else if (p0.qk_heads > 0)
-      fp8_gemm_kernel<false, true, 2, 4><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
-    else
-      fp8_gemm_kernel<false, false, 2, 4><<<dim3((unsigned)grid), dim3(256), kMainLdsBytes, st>>>(q);
+    launch_form<2>(q, p0, ext, grid, st);
     return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
   }
   const int grid = ((q.total + 7) / 8) * 8;
-  if (p0.resid)
-    fp8_gemm_kernel<true, false, 4, 4><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
-  else if (p0.qk_heads > 0)
-    fp8_gemm_kernel<false, true, 4, 4><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
-  else
-    fp8_gemm_kernel<false, false, 4, 4><<<dim3((unsigned)grid), dim3(512), kMainLdsBytes, st>>>(q);
+  launch_form<4>(q, p0, ext, grid, st);
   return hipGetLastError() == hipSuccess ? DSX_OK : DSX_ELAUNCH;
 }
 
@@ -898,6 +944,9 @@ static int gemm_fill(dsx::GemmArgs& p, const void* a, int64_t lda, const void* w
   p.rope_sb = 0;
   p.rope_pos0 = p.qk_heads = 0;
   p.qk_eps = 0.f;
+  p.a2 = p.w2 = nullptr;
+  p.lda2 = p.ldw2 = 0;
+  p.K2 = 0;
   return DSX_OK;
 }
 
@@ -976,6 +1025,20 @@ static int problem_fill(dsx::GemmArgs& p, const dsx_gemm_problem& d) {
     p.qk_heads = d.qk_heads;
     p.qk_eps = d.norm_eps;
     p.rows_per_batch = (int)d.rows_per_batch;
+    if (!gemm_main_kernel_ok(p)) return DSX_EBADSHAPE;
+  }
+  if (d.K_ext != 0) {
+    // the second segment of the reduction axis exists in the tile kernel only; its unit count and the kernel's
+    // prologue (two units of the first segment) bound the shapes
+    if (d.K_ext < 0 || d.K_ext > (1 << 30) || (d.K_ext % 128) || d.K < 256 || d.M <= 0) return DSX_EBADSHAPE;
+    if (!d.a_ext || !d.w_ext) return DSX_ENULL;
+    if (d.lda_ext < d.K_ext || d.ldw_ext < d.K_ext || d.lda_ext >= (1 << 24) || d.ldw_ext >= (1 << 24)) return DSX_EBADSHAPE;
+    if ((d.lda_ext & 15) || (d.ldw_ext & 15) || ((uintptr_t)d.a_ext & 15) || ((uintptr_t)d.w_ext & 15)) return DSX_EALIGN;
+    p.a2 = (const uint8_t*)d.a_ext;
+    p.w2 = (const uint8_t*)d.w_ext;
+    p.lda2 = d.lda_ext;
+    p.ldw2 = d.ldw_ext;
+    p.K2 = (int)d.K_ext;
     if (!gemm_main_kernel_ok(p)) return DSX_EBADSHAPE;
   }
   return DSX_OK;

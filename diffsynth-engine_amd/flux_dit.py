@@ -49,9 +49,20 @@ def _lora_factors(down: torch.Tensor, up: torch.Tensor, coef: float, n: int, k: 
 
 
 class _Linear:
-    """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias, plus optional unfused LoRA pairs."""
+    """An e4m3 weight (N,K) with its per-tensor scale and bf16 bias, plus optional unfused LoRA pairs.
 
-    __slots__ = ("w", "s", "b", "n", "k", "loras", "scaled", "prequantised")
+    Unfused low-rank updates (LoRALinear.forward, models/basic/lora.py:29-32,137-141: y += c * up(down(x))) ride the
+    main product as 128 more columns of its reduction axis whenever the layer runs on the tile kernel in scaled mode:
+    ``t = down(x)`` comes from one small HBM-bound kernel (ops.lora_down) as e4m3 on the row's own scale grid, and
+    ``c * up / s_w`` is stored next to the weight as the matching 128 columns (each rank repeated as often as 128
+    columns allow, every copy carrying its share of t), so that
+    ``s_x[m] s_w (sum_k xq wq + sum_r t u) = x W^T + c up(down(x))`` comes out of ONE accumulation with every
+    epilogue (bias, gated residual, q/k RMSNorm + RoPE) unchanged.  Elsewhere (unit-scale mode, whose arithmetic is
+    the reference's bare casts with the coefficient applied in bf16; products with at most 8 rows; ranks beyond 128;
+    updates so strong that t would leave e4m3's range)
+    the update is two more products added through residual epilogues."""
+
+    __slots__ = ("w", "s", "b", "n", "k", "loras", "scaled", "prequantised", "_raw", "_ext")
 
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], scaled: bool):
         self.prequantised = weight.dtype == ops.FP8
@@ -61,31 +72,78 @@ class _Linear:
             self.w, self.s = ops.quantize_weight_fp8(weight, scaled=scaled)
         self.b = None if bias is None else bias.to(torch.bfloat16).contiguous()
         self.n, self.k = self.w.shape
-        self.loras = []  # (down_q (r,K), down_scale, up_q (N,r), up_scale * coefficient)
+        self.loras = []  # (down_q (r,K), down_scale, up_q (N,r), up_scale * coefficient): the two-product form
+        self._raw = []   # (down, up, coefficient) as given: the extension form is built from these on first use
+        self._ext = None
         self.scaled = scaled
 
     def add_lora(self, down: torch.Tensor, up: torch.Tensor, coef: float):
         """Unfused low-rank update y += coef * up(down(x)) (models/basic/lora.py:29-32,137-141); both factors are
-        stored as e4m3 like every other Linear under fp8 inference.  The rank is zero-padded (see _lora_factors)
-        and the coefficient is folded into the up factor's scale."""
+        stored as e4m3 like every other Linear under fp8 inference."""
         self.loras.append(_lora_factors(down, up, coef, self.n, self.k, self.w.device))
+        self._raw.append((down, up, float(coef)))
+        self._ext = None
+
+    def _extension(self):
+        """(stacked down factors e4m3 (R,K), per-row scale fp32 (R), extension weight e4m3 (N,128), copies, columns per copy) or None when
+        the updates of this layer do not fit the extension form."""
+        if self._ext is None:
+            dev, f32 = self.w.device, torch.float32
+            total = sum(d.shape[0] for d, _, _ in self._raw)
+            if self.s is None or total > 128 or self.k % 128 or self.k < 256 or self.n % 8:
+                self._ext = False
+            else:
+                # Every rank is laid down `copies` times, each copy carrying 1 / copies of t: the few terms of a
+                # low-rank product would otherwise have to be as large, each, as the sum of K terms they sit beside,
+                # and e4m3 ends at 448.  The 128 columns are there anyway.
+                ranks = (total + 3) // 4 * 4   # columns of one copy (written four at a time)
+                R = (total + 31) // 32 * 32    # rows of the stacked down factors (whole MFMA tiles)
+                copies = min(128 // ranks, 32)
+                d_all = torch.zeros((R, self.k), dtype=ops.FP8, device=dev)
+                rs = torch.zeros((R,), dtype=f32, device=dev)
+                u_all = torch.zeros((self.n, 128), dtype=ops.FP8, device=dev)
+                r0, fits = 0, True
+                for down, up, coef in self._raw:
+                    r = down.shape[0]
+                    dq, ds = ops.quantize_weight_fp8(down.to(dev, torch.bfloat16).contiguous(), scaled=True)
+                    # what the main product's scales leave to be multiplied in: c * up / s_w, on its own e4m3 grid
+                    uq, us = ops.quantize_weight_fp8((up.to(dev, f32) * coef / self.s).contiguous(), scaled=True)
+                    d_all[r0:r0 + r] = dq
+                    rs[r0:r0 + r] = ds * us / copies
+                    for c in range(copies):
+                        u_all[:, c * ranks + r0:c * ranks + r0 + r] = uq
+                    r0 += r
+                    # t of a row of N(0,1)-like codes (rms 448 / 4) against the longest down row, four deviations
+                    # out, has to stay inside e4m3; an update too strong for that takes the two-product form
+                    t_far = 4.0 * 112.0 * dq.float().norm(dim=1).max() * ds * us / copies
+                    fits = fits and bool(t_far <= 448.0)
+                self._ext = (d_all, rs, u_all, copies, ranks) if fits else False
+        return self._ext or None
+
+    def _rides_main_product(self, a_q) -> bool:
+        return bool(self.loras) and a_q.shape[0] > 8 and self._extension() is not None
 
     def problem(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None, qk=None):
-        """Keyword arguments of ``ops.fp8_gemm`` for this layer applied to ``a_q``."""
+        """Keyword arguments of ``ops.fp8_gemm`` for this layer applied to ``a_q`` (low-rank updates included when
+        they ride the main product: their down projection is launched here)."""
+        ext = None
+        if self._rides_main_product(a_q):
+            d_all, rs, u_all, copies, ranks = self._extension()
+            ext = (ops.lora_down(a_q, d_all, rs, 128, copies, ranks), u_all)
         return dict(a_q=a_q, w_q=self.w, a_scale=a_s if self.s is not None else None, w_scale=self.s, bias=self.b,
-                    out=out, resid=resid, gate=gate, rows_per_batch=rows_per_batch, qk=qk)
+                    out=out, resid=resid, gate=gate, rows_per_batch=rows_per_batch, qk=qk, ext=ext)
 
     def __call__(self, a_q, a_s, out=None, resid=None, gate=None, rows_per_batch=None, qk=None):
-        if not self.loras:
+        if not self.loras or self._rides_main_product(a_q):
             return ops.fp8_gemm(**self.problem(a_q, a_s, out, resid, gate, rows_per_batch, qk))
         if qk is not None:  # the low-rank terms are added after the main product: q/k can only be prepared after them
             raise ValueError("a LoRA on a qkv projection needs qk_prep='attention'")
+        main = dict(a_q=a_q, w_q=self.w, a_scale=a_s if self.s is not None else None, w_scale=self.s, bias=self.b)
         if resid is None:  # y = main + sum(lora): the low-rank products are added by residual epilogues
             # the main product and the first down projection read the same operand and have the same (plain)
             # epilogue: one launch, in which the few tiles of the projection run beside the main product's
             dq, ds, _, _ = self.loras[0]
-            y, h0 = ops.fp8_gemm_grouped([self.problem(a_q, a_s, out),
-                                          dict(a_q=a_q, w_q=dq, a_scale=a_s, w_scale=ds, bias=None)])
+            y, h0 = ops.fp8_gemm_grouped([dict(main, out=out), dict(a_q=a_q, w_q=dq, a_scale=a_s, w_scale=ds, bias=None)])
             hs_list = [h0] + [ops.fp8_gemm(a_q, dq, a_s, ds, None) for dq, ds, _, _ in self.loras[1:]]
             for h, (_, _, uq, us) in zip(hs_list, self.loras):
                 hq, hs = ops.quantize_fp8(h, scaled=True)
@@ -99,12 +157,13 @@ class _Linear:
         acc = resid
         for hq, hs, uq, us in lows:
             acc = ops.fp8_gemm(hq, uq, hs, us, None, resid=acc, gate=gate, rows_per_batch=rows_per_batch)
-        return ops.fp8_gemm(**self.problem(a_q, a_s, out, acc, gate, rows_per_batch))
+        return ops.fp8_gemm(**dict(main, out=out, resid=acc, gate=gate, rows_per_batch=rows_per_batch))
 
 
 def _gemm_pair(la: "_Linear", pa: dict, lb: "_Linear", pb: dict):
-    """Two independent linears (image and text stream): one grouped submission unless a LoRA is attached."""
-    if la.loras or lb.loras:
+    """Two independent linears (image and text stream): one grouped submission, unless one of them carries low-rank
+    updates in the two-product form."""
+    if any(L.loras and not L._rides_main_product(p["a_q"]) for L, p in ((la, pa), (lb, pb))):
         return la(**pa), lb(**pb)
     return ops.fp8_gemm_grouped([la.problem(**pa), lb.problem(**pb)])
 
@@ -254,11 +313,11 @@ class FluxDiTRunner:
         self.lin[name].add_lora(down, up, coef)
 
     def _qk_in_gemm(self, rows, *layers) -> bool:
-        """q/k are prepared in the GEMM epilogue unless a LoRA rides on one of the projections (its low-rank
-        terms are added after the main product, so the projection is complete only after them) or a problem is
+        """q/k are prepared in the GEMM epilogue unless a projection carries low-rank updates in the two-product
+        form (added after the main product, so the projection is complete only after them) or a problem is
         outside what the tile kernel that carries the epilogue takes (more than 8 rows, K a multiple of 128)."""
-        return (self.qk_prep == "gemm" and not any(L.loras for L in layers) and min(rows) > 8
-                and all(L.k % 128 == 0 and L.n % 8 == 0 for L in layers))
+        return (self.qk_prep == "gemm" and not any(L.loras and L._extension() is None for L in layers)
+                and min(rows) > 8 and all(L.k % 128 == 0 and L.n % 8 == 0 for L in layers))
 
     # ------------------------------------------------------------------ small helpers
     def _linear_bf16(self, x: torch.Tensor, name: str) -> torch.Tensor:

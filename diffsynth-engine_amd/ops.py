@@ -87,7 +87,7 @@ def quantize_weight_fp8(w: torch.Tensor, scaled: bool = True):
 
 
 def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, resid=None, gate=None,
-                  rows_per_batch=None, qk=None):
+                  rows_per_batch=None, qk=None, ext=None):
     """Validate one GEMM and describe it as a ``dsx_gemm_problem``; returns (problem, out, keep-alive refs).
 
     ``qk``: optional dict(heads=H, q_norm_w=, k_norm_w=, rope=(B|1, S, 64, 2) fp32 table or None, pos0=, eps=) for a
@@ -163,21 +163,34 @@ def _gemm_problem(a_q, w_q, a_scale=None, w_scale=None, bias=None, out=None, res
             prob.rope_sb = rope.stride(0) if rope.shape[0] > 1 else 0
             prob.rope_pos0 = int(qk.get("pos0", 0))
         keep += [wq, wk, rope]
+    if ext is not None:
+        # (a_ext (M, K_ext), w_ext (N, K_ext)): more columns of the reduction axis, e.g. an unfused low-rank update
+        a_e, w_e = ext
+        _require_cuda(a_e, w_e)
+        if a_e.dtype != FP8 or w_e.dtype != FP8 or a_e.dim() != 2 or w_e.dim() != 2 or a_e.shape[0] != M \
+                or w_e.shape[0] != N or a_e.shape[1] != w_e.shape[1] or a_e.stride(1) != 1 or w_e.stride(1) != 1:
+            raise ValueError("fp8_gemm: `ext` must be e4m3 (M, K_ext) and (N, K_ext) with unit column stride")
+        prob.a_ext, prob.lda_ext, prob.w_ext, prob.ldw_ext = _ptr(a_e), a_e.stride(0), _ptr(w_e), w_e.stride(0)
+        prob.K_ext = a_e.shape[1]
+        keep += [a_e, w_e]
     return prob, out, tuple(keep)
 
 
 def fp8_gemm(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor] = None,
              w_scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
              out: Optional[torch.Tensor] = None, resid: Optional[torch.Tensor] = None,
-             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None, qk=None) -> torch.Tensor:
+             gate: Optional[torch.Tensor] = None, rows_per_batch: Optional[int] = None, qk=None,
+             ext=None) -> torch.Tensor:
     """out[m,n] = bf16((sum_k a[m,k] w[n,k]) * a_scale[m] * w_scale + bias[n]); a (M,K), w (N,K) e4m3.
 
     With ``resid`` (M,N) the gated residual is fused: out = resid + gate * that, gate (B,N) or None,
     rows_per_batch = rows of a per batch entry (default: all M rows share gate row 0).
-    With ``qk`` (see _gemm_problem) the q and k heads of a packed qkv projection leave normalised and rotated."""
-    if qk is not None:
+    With ``qk`` (see _gemm_problem) the q and k heads of a packed qkv projection leave normalised and rotated.
+    With ``ext`` = (a_ext (M,E), w_ext (N,E)) the sum runs over E more columns, as if a and w were [a | a_ext] and
+    [w | w_ext]."""
+    if qk is not None or ext is not None:  # options the problem description carries and the flat entry points do not
         return fp8_gemm_grouped([dict(a_q=a_q, w_q=w_q, a_scale=a_scale, w_scale=w_scale, bias=bias, out=out,
-                                      rows_per_batch=rows_per_batch, qk=qk)])[0]
+                                      resid=resid, gate=gate, rows_per_batch=rows_per_batch, qk=qk, ext=ext)])[0]
     pr, out, _keep = _gemm_problem(a_q, w_q, a_scale, w_scale, bias, out, resid, gate, rows_per_batch)
     lib = _lib.load()
     if resid is None:
@@ -203,6 +216,27 @@ def fp8_gemm_grouped(problems):
     rc = _lib.load().dsx_fp8_gemm_grouped(arr, len(built), _stream())
     _lib.check(rc, "dsx_fp8_gemm_grouped")
     return [b[1] for b in built]
+
+
+def lora_down(a_q: torch.Tensor, d_q: torch.Tensor, row_scale: torch.Tensor, width: int = 128, copies: int = 1,
+              ranks: Optional[int] = None) -> torch.Tensor:
+    """(M, width) e4m3: columns c ranks + r (r < ranks, c < copies) hold
+    e4m3_saturating(row_scale[r] * sum_k a_q[m,k] d_q[r,k]), the rest zero codes; the operand `ext` of :func:`fp8_gemm`
+    for an unfused low-rank update.  d_q: the stacked down factors, zero rows from `ranks` (default: all) up to
+    R = d_q.shape[0], a multiple of 32 and at most 128."""
+    _require_cuda(a_q, d_q, row_scale)
+    if a_q.dtype != FP8 or d_q.dtype != FP8 or a_q.dim() != 2 or d_q.dim() != 2 or a_q.shape[1] != d_q.shape[1] \
+            or a_q.stride(1) != 1 or not d_q.is_contiguous():
+        raise ValueError("lora_down expects e4m3 a (M,K) and contiguous d (R,K)")
+    M, K = a_q.shape
+    R = d_q.shape[0]
+    if row_scale.dtype != torch.float32 or row_scale.numel() != R or not row_scale.is_contiguous():
+        raise ValueError("lora_down: row_scale must hold one contiguous fp32 value per row of d")
+    out = torch.empty((M, width), dtype=FP8, device=a_q.device)
+    rc = _lib.load().dsx_lora_down(_ptr(a_q), a_q.stride(0), _ptr(d_q), K, _ptr(row_scale), _ptr(out), width, M, K, R,
+                                   R if ranks is None else ranks, copies, width, _stream())
+    _lib.check(rc, "dsx_lora_down")
+    return out
 
 
 def fp8_gemv_rowscale(a_q: torch.Tensor, w_q: torch.Tensor, a_scale: Optional[torch.Tensor],

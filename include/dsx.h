@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define DSX_ABI_VERSION 6
+#define DSX_ABI_VERSION 7
 
 enum {
   DSX_OK = 0,
@@ -138,8 +138,35 @@ typedef struct dsx_gemm_problem {
   const float* rope; int64_t rope_sb, rope_pos0, rope_rows;
   float norm_eps;
   int32_t qk_heads;
+  /* Optional extension of the reduction axis (K_ext > 0): the product runs over the K columns of (a, w) followed by
+   * the K_ext columns of (a_ext, w_ext), as if the operands were the concatenations [a | a_ext] (M, K + K_ext) and
+   * [w | w_ext] (N, K + K_ext), without either concatenation existing; one accumulation, one pair of scales, every
+   * epilogue as usual.  This is how an unfused low-rank update rides the main product (dsx_lora_down writes a_ext;
+   * LoRALinear.forward, models/basic/lora.py:29-32,137-141).  K_ext % 128 == 0, K >= 256, and the shape the
+   * 256x256-tile kernel takes (as for qk_heads), DSX_EBADSHAPE otherwise. */
+  const void* a_ext; int64_t lda_ext;  /* (M,K_ext) e4m3 */
+  const void* w_ext; int64_t ldw_ext;  /* (N,K_ext) e4m3 */
+  int64_t K_ext;
 } dsx_gemm_problem;
 int dsx_fp8_gemm_grouped(const dsx_gemm_problem* problems, int count, void* stream);
+
+/*
+ * Down projection of unfused low-rank updates, written as the extension operand of the main product
+ * (dsx_gemm_problem.a_ext): out[m, c ranks + r] = e4m3_saturating(row_scale[r] * sum_k a[m,k] d[r,k]) for
+ * r < ranks and c < copies, zero codes from column copies * ranks up to E.  a (M,K) e4m3 codes of the activation (its
+ * per-token scale is applied later, by the main product, to the whole extended sum), d (R,K) e4m3: the down factors
+ * of every update on the layer stacked row-wise and zero-padded from row `ranks` to R, row_scale (R) fp32: per
+ * stacked row the product of its factor's quantisation scale and of whatever the caller folded into the matching
+ * columns of w_ext (1 / copies included: writing a row's values `copies` times, against as many repeats of w_ext's
+ * columns, keeps each of them that much further from e4m3's end).
+ * R % 32 == 0, R <= 128, ranks % 4 == 0, ranks <= R, 1 <= copies <= 32, E >= copies * ranks, E % 16 == 0,
+ * K % 64 == 0.
+ * Replaces `lora.down(x)` of LoRA.forward (diffsynth_engine/models/basic/lora.py:29-32) for every update of a layer
+ * in one HBM-bound pass over a.
+ */
+int dsx_lora_down(const void* a, int64_t lda, const void* d, int64_t ldd, const float* row_scale, void* out,
+                  int64_t ldo, int64_t M, int64_t K, int64_t R, int64_t ranks, int64_t copies, int64_t E,
+                  void* stream);
 
 /*
  * Small-M (M <= 8) form of dsx_fp8_gemm with one weight scale PER OUTPUT ROW (w_row_scale[n]), so that

@@ -32,7 +32,7 @@ def test_abi_version_and_strerror():
     from diffsynth_engine_amd import _lib
 
     lib = _lib.load()
-    assert lib.dsx_abi_version() == 6
+    assert lib.dsx_abi_version() == 7
     assert _lib.strerror(0) == "ok"
     for code in (-1, -2, -3, -4, -5, -6):
         assert _lib.strerror(code) and "unknown" not in _lib.strerror(code)
@@ -256,7 +256,7 @@ def test_gemm_problem_struct_layout_and_qk_epilogue_checks():
     than 2 * heads * 128, with a RoPE table that ends before the last token's row, and outside the tile kernel's shapes."""
     from diffsynth_engine_amd import _lib
 
-    assert ctypes.sizeof(_lib.GemmProblem) == 17 * 8 + 2 * 8 + 8 + 3 * 8 + 4 + 4
+    assert ctypes.sizeof(_lib.GemmProblem) == 17 * 8 + 2 * 8 + 8 + 3 * 8 + 4 + 4 + 5 * 8
     lib = _lib.load()
     buf = ctypes.create_string_buffer(1 << 12)
     p16 = (ctypes.addressof(buf) + 15) & ~15

@@ -296,8 +296,13 @@ def test_unfused_lora_on_runner_linears(dev):
                "blocks.0.norm1_a.linear": 8, "single_blocks.0.norm.linear": 16}
     for name, r in targets.items():
         n, k = sd[name + ".weight"].shape
-        down = (torch.randn(r, k, generator=g) * 0.05).bfloat16()
-        up = (torch.randn(n, r, generator=g) * 0.05).bfloat16()
+        # (an update of ~10 % of the layer's own output: strong for a LoRA, and enough to matter below.  The runner
+        # carries it as an extension of the main product's reduction axis, the oracle as LoRALinear.forward's two
+        # further linears: two quantisations of one update, each as close to the exact update as the other --
+        # test_lora_forms_are_equally_close_to_the_exact_update -- whose difference the block's later quantisers
+        # amplify like any other perturbation)
+        down = (torch.randn(r, k, generator=g) * 0.03).bfloat16()
+        up = (torch.randn(n, r, generator=g) * 0.03).bfloat16()
         P.lora[name] = [(down, up, 0.5)]
         R.add_lora(name, down, up, 0.5)
     St, side = 40, 12
@@ -324,3 +329,43 @@ def test_unfused_lora_on_runner_linears(dev):
     want = oflux.single_block(P, 0, x, cond, freqs)
     got = R._single_block(0, x.to(dev), mods["single_blocks.0.norm.linear"], rope)
     assert _cos(got, want) >= 0.9995, _cos(got, want)
+
+
+@pytest.mark.parametrize("M,K,N,r,std,coef", [(4608, 3072, 9216, 16, 0.05, 0.5), (4608, 3072, 9216, 16, 0.01, 0.5),
+                                              (4608, 15360, 3072, 4, 0.05, 0.5), (512, 3072, 3072, 64, 0.02, 1.0),
+                                              (600, 1024, 512, 100, 0.02, 1.0)])
+def test_lora_forms_are_equally_close_to_the_exact_update(dev, M, K, N, r, std, coef):
+    """An unfused low-rank update in its two forms -- 128 more columns of the main product's reduction axis
+    (ops.lora_down + dsx_gemm_problem.a_ext), and LoRALinear.forward's two further products added through residual
+    epilogues -- against x W^T + c (x D^T) U^T evaluated in fp32 on the dequantised operands and the unquantised
+    factors: both within 1e-4 of cosine 1 for updates from 1 % to 25 % of the layer's output, neither behind the
+    other by more than 1e-5, and the update itself (output minus main product) recovered to 0.97 and better."""
+    from diffsynth_engine_amd import ops
+    from diffsynth_engine_amd.flux_dit import _Linear
+
+    g = torch.Generator().manual_seed(M + K + r)
+    x = torch.randn(M, K, generator=g).bfloat16().to(dev)
+    W = (torch.randn(N, K, generator=g) * 0.02).bfloat16().to(dev)
+    D = (torch.randn(r, K, generator=g) * std).bfloat16().to(dev)
+    U = (torch.randn(N, r, generator=g) * std).bfloat16().to(dev)
+    xq, xs = ops.quantize_fp8(x)
+    rides = _Linear(W, None, True)
+    rides.add_lora(D, U, coef)
+    assert rides._extension() is not None
+    two = _Linear(W, None, True)
+    two.add_lora(D, U, coef)
+    two._ext = False
+    y_ext, y_two = rides(xq, xs), two(xq, xs)
+    xd, wd = xq.float() * xs[:, None], rides.w.float() * rides.s
+    main = xd @ wd.t()
+    lora = coef * ((xd @ D.float().t()) @ U.float().t())
+    c_ext, c_two = _cos(y_ext, main + lora), _cos(y_two, main + lora)
+    assert c_ext >= 0.9999 and c_two >= 0.9999 and c_ext >= c_two - 1e-5, (c_ext, c_two)
+    assert _cos(y_ext.float() - main, lora) >= 0.97
+    # a rank beyond 128, or an update whose down projection would leave e4m3's range, keeps the two-product form
+    big = _Linear(W, None, True)
+    big.add_lora(torch.cat([D] * (128 // r + 1)), torch.cat([U] * (128 // r + 1), dim=1), coef)
+    assert big._extension() is None
+    strong = _Linear(W, None, True)
+    strong.add_lora(D * 64, U, coef)
+    assert strong._extension() is None

@@ -334,3 +334,92 @@ def test_half_height_tiles_give_the_bits_of_full_tiles(dev, kind):
         elif kind == "qk":
             kws = dict(rows_per_batch=m, qk=kw_big["qk"])
         assert torch.equal(ops.fp8_gemm(xq[:m], w8, xs[:m], ws, bias, **kws), big[:m]), m
+
+
+@pytest.mark.parametrize("kind", ["plain", "residual", "qk"])
+@pytest.mark.parametrize("M", [4608, 700])
+def test_k_extension_equals_the_concatenated_operands(dev, kind, M):
+    """dsx_gemm_problem.a_ext / w_ext: K_ext more columns of the reduction axis read from operands of their own.
+    The units are consumed in the order the concatenations [a | a_ext], [w | w_ext] would give, so the result is
+    the concatenated product's bit for bit, with each epilogue, on 256-row and on 128-row tiles."""
+    from diffsynth_engine_amd import ops
+
+    K, E, N, heads = 1024, 128, 1536, 4
+    g = torch.Generator().manual_seed(M + len(kind))
+    x = torch.randn(M, K + E, generator=g).bfloat16().to(dev)
+    w = (torch.randn(N, K + E, generator=g) * 0.05).bfloat16().to(dev)
+    bias = torch.randn(N, generator=g).bfloat16().to(dev)
+    w8, ws = ops.quantize_weight_fp8(w)
+    xq, xs = ops.quantize_fp8(x)
+    kw = {}
+    if kind == "residual":
+        kw = dict(resid=torch.randn(M, N, generator=g).bfloat16().to(dev),
+                  gate=torch.randn(1, N, generator=g).bfloat16().to(dev), rows_per_batch=M)
+    elif kind == "qk":
+        ang = torch.rand(1, M, 64, generator=g) * 6.28
+        rope = torch.stack((torch.cos(ang), torch.sin(ang)), dim=-1).float().to(dev)
+        nq, nk = [(1 + 0.2 * torch.randn(128, generator=g)).bfloat16().to(dev) for _ in range(2)]
+        kw = dict(rows_per_batch=M, qk=dict(heads=heads, q_norm_w=nq, k_norm_w=nk, rope=rope, pos0=0, eps=1e-6))
+    whole = ops.fp8_gemm(xq, w8, xs, ws, bias, **kw)
+    # the two segments as separate allocations with leading dimensions of their own
+    a1, a2 = xq[:, :K].contiguous(), xq[:, K:].contiguous()
+    w1, w2 = w8[:, :K].contiguous(), w8[:, K:].contiguous()
+    split = ops.fp8_gemm(a1, w1, xs, ws, bias, ext=(a2, w2), **kw)
+    assert torch.equal(split, whole)
+    # and it is the extension that closes the gap
+    assert not torch.equal(ops.fp8_gemm(a1, w1, xs, ws, bias, **kw), whole)
+
+
+def test_k_extension_refusals(dev):
+    from diffsynth_engine_amd import ops
+
+    a, w = torch.zeros(64, 256, device=dev).to(ops.FP8), torch.zeros(64, 256, device=dev).to(ops.FP8)
+    e = lambda m, k: torch.zeros(m, k, device=dev).to(ops.FP8)
+    with pytest.raises(ValueError):
+        ops.fp8_gemm(a, w, ext=(e(64, 64), e(64, 64)))       # K_ext % 128
+    with pytest.raises(ValueError):
+        ops.fp8_gemm(a, w, ext=(e(63, 128), e(64, 128)))     # rows of a_ext
+    with pytest.raises(ValueError):
+        ops.fp8_gemm(a[:, :128], w[:, :128], ext=(e(64, 128), e(64, 128)))  # the first segment needs two units
+    with pytest.raises(ValueError):
+        ops.fp8_gemm(a[:8], w, ext=(e(8, 128), e(64, 128)))  # the small-M kernel has no extension
+
+
+@pytest.mark.parametrize("M,K,R", [(4608, 3072, 32), (4608, 15360, 64), (515, 1024, 128), (40, 256, 96)])
+def test_lora_down_against_the_fp32_product(dev, M, K, R):
+    """out[m, c R + r] = e4m3_saturating(row_scale[r] * sum_k a[m,k] d[r,k]) for every copy c, zero codes after the
+    last copy.  The products
+    of e4m3 codes are exact in fp32; the kernel's sum is split over wavefronts, so it may differ from torch's in the
+    last bit and a value that sits on a rounding boundary may land on the neighbouring code: at most a handful of
+    codes differ, each by one step."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(M + K + R)
+    a = torch.randn(M, K, generator=g).mul(60).to(dev).to(ops.FP8)
+    d = torch.randn(R, K, generator=g).mul(60).to(dev).to(ops.FP8)
+    rs = (torch.rand(R, generator=g) + 0.5).mul(3e-5).to(dev)
+    rs[R - 1] = 1.0  # one column far beyond 448: saturates instead of turning into NaN codes
+    copies = 128 // R if M > 100 else 1
+    got = ops.lora_down(a, d, rs, 128, copies)
+    assert got.shape == (M, 128) and got.dtype == ops.FP8
+    for c in range(1, copies):  # every copy is the first one again
+        assert torch.equal(got[:, c * R:(c + 1) * R].view(torch.uint8), got[:, :R].view(torch.uint8))
+    # fewer valid ranks than rows of d (the rest is padding): narrower copies, more of them
+    few = ops.lora_down(a, d, rs, 128, 128 // 12, ranks=12)
+    for c in range(128 // 12):
+        assert torch.equal(few[:, c * 12:(c + 1) * 12].view(torch.uint8), got[:, :12].view(torch.uint8))
+    assert (few[:, 120:].view(torch.uint8) == 0).all()
+    ref = ((a.double() @ d.double().t()) * rs.double()).float()  # (fp32 matmul of 15360 terms is itself off by ~1)
+    want = ref.clamp(-448, 448).to(ops.FP8)
+    gf, wf = got[:, :R].float(), want.float()
+    assert torch.isfinite(gf).all()
+    assert (gf[:, R - 1].abs() == 448).float().mean().item() > 0.98  # (a sum can land inside the range by chance)
+    differ = gf != wf
+    assert differ.float().mean().item() < 2e-3
+    # a differing code is the other neighbour of the exact value on the grid: never further than one step.  (Not
+    # asked of the saturating column: its scale of 1 lays bare the absolute error of a sum of 15 360 products of up to
+    # 2e5 each -- the matrix pipe's fp32 accumulation is good to about 1e-5 of the partial sums' magnitude, which a
+    # scale that brings typical values into e4m3's range makes invisible.)
+    step = wf.abs().clamp_min(2 ** -6) * 0.125
+    assert ((gf - ref.clamp(-448, 448)).abs() <= step)[:, : R - 1].all()
+    assert (got[:, copies * R:].view(torch.uint8) == 0).all()
