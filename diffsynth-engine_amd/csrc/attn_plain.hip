@@ -626,21 +626,6 @@ static int64_t plan_split(const dsx_attn_params& p, int cus, AttnSplit& sp) {
   return (int64_t)tail * sp.max_parts * kSlotFloats * (int64_t)sizeof(float);
 }
 
-// Compute units of the current device (0 when it cannot be asked).
-static int device_cus() {
-  static PerDeviceOnce once;
-  static int cus[kMaxDevices];
-  int dev = -1;
-  const int rc = per_device_once(once, [&](int d) {
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, d) != hipSuccess) return (int)DSX_EARCH;
-    cus[d] = prop.multiProcessorCount;
-    return (int)DSX_OK;
-  });
-  if (rc != DSX_OK || hipGetDevice(&dev) != hipSuccess) return 0;
-  return cus[dev];
-}
-
 int64_t attn_plain_workspace_bytes(const dsx_attn_params& p) {
   AttnSplit sp;
   return plan_split(p, device_cus(), sp);

@@ -28,6 +28,21 @@ inline int per_device_once(PerDeviceOnce& once, F&& init) {
   return rc;
 }
 
+// Compute units of the current device (0 when it cannot be asked).
+inline int device_cus() {
+  static PerDeviceOnce once;
+  static int cus[kMaxDevices];
+  int dev = -1;
+  const int rc = per_device_once(once, [&](int d) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, d) != hipSuccess) return (int)DSX_EARCH;
+    cus[d] = prop.multiProcessorCount;
+    return (int)DSX_OK;
+  });
+  if (rc != DSX_OK || hipGetDevice(&dev) != hipSuccess) return 0;
+  return cus[dev];
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -64,6 +79,21 @@ __device__ __forceinline__ void round_bf16_pair(float& a, float& b) {
   const uint32_t w = pack_bf16x2(a, b);
   a = __uint_as_float(w << 16);
   b = __uint_as_float(w & 0xffff0000u);
+}
+
+// The same, with the conversion kept as ONE instruction: left to itself the compiler splits the pair into two
+// single conversions (each with its own shift and mask) wherever the two halves are used apart.
+__device__ __forceinline__ void round_bf16_pair_fused(float& a, float& b) {
+  uint32_t w;
+  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));
+  a = __uint_as_float(w << 16);
+  b = __uint_as_float(w & 0xffff0000u);
+}
+// max(m, |a|, |b|) in one instruction (the compiler spends two more on canonicalising |a| and |b|).
+__device__ __forceinline__ float max3_abs(float m, float a, float b) {
+  float r;
+  asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(m), "v"(a), "v"(b));
+  return r;
 }
 
 // Unpack the two bf16 halves of a 32-bit word.

@@ -83,7 +83,7 @@ __device__ __forceinline__ void emit_row(float (&val)[NCH][8], int nchunk, uint1
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(val[i][j]));
+      for (int j = 0; j < 8; j += 2) amax = max3_abs(amax, val[i][j], val[i][j + 1]);
     }
     amax = fmaxf(row_max<TPR>(amax, red), 1e-12f);
     const float inv = 448.0f / amax;
@@ -180,17 +180,17 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
     // every bf16 tensor of the separate ops is a rounding point: LayerNorm output, 1 + scale, the product,
     // the sum; roundings go in pairs through one conversion
 #pragma unroll
-    for (int j = 0; j < 8; j += 2) round_bf16_pair(v[j], v[j + 1]);
+    for (int j = 0; j < 8; j += 2) round_bf16_pair_fused(v[j], v[j + 1]);
     if (sc) {
       float s8[8];
       unpack8(sraw[i], s8);
 #pragma unroll
       for (int j = 0; j < 8; j += 2) {
         float a = 1.0f + s8[j], b = 1.0f + s8[j + 1];
-        round_bf16_pair(a, b);
+        round_bf16_pair_fused(a, b);
         v[j] *= a;
         v[j + 1] *= b;
-        round_bf16_pair(v[j], v[j + 1]);
+        round_bf16_pair_fused(v[j], v[j + 1]);
       }
     }
     if (sh) {
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
       for (int j = 0; j < 8; j += 2) {
         v[j] += h8[j];
         v[j + 1] += h8[j + 1];
-        round_bf16_pair(v[j], v[j + 1]);
+        round_bf16_pair_fused(v[j], v[j + 1]);
       }
     }
 #pragma unroll
@@ -215,6 +215,83 @@ __global__ __launch_bounds__(256) void adaln_modulate_kernel(
   if (!live && TPR == 64) return;  // wave-uniform; wider row slots share the workgroup's barriers
   emit_row<NCH, TPR>(val, nchunk, y ? y + row * ldy : nullptr, q ? q + row * ldq : nullptr, q_scale, row,
                      red, live);
+}
+
+// The form of adaln_modulate_kernel<NCH, 64> the DiT step launches a hundred times: rows of exactly NCH * 512
+// values, both modulation vectors, no LayerNorm affine, e4m3 output with its per-token scale and nothing else.  With
+// every option fixed at compile time the row is one straight line of code; the arithmetic and its order are those of
+// the general kernel (same bits out).
+template <int NCH>
+__global__ __launch_bounds__(256) void adaln_quant_rows_kernel(
+    const uint16_t* __restrict__ x, int64_t ldx, const uint16_t* __restrict__ scale,
+    const uint16_t* __restrict__ shift, int64_t mod_sb, int64_t rows_per_batch, float eps,
+    uint8_t* __restrict__ q, int64_t ldq, float* __restrict__ q_scale, int64_t rows) {
+  const int t = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;  // wave-uniform; the kernel has no barrier
+  const u32x4* xr = reinterpret_cast<const u32x4*>(x + row * ldx);
+  const int64_t bidx = row / rows_per_batch;
+  const u32x4* sc = reinterpret_cast<const u32x4*>(scale + bidx * mod_sb);
+  const u32x4* sh = reinterpret_cast<const u32x4*>(shift + bidx * mod_sb);
+  u32x4 raw[NCH], sraw[NCH], hraw[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) raw[i] = xr[t + i * 64];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) sraw[i] = sc[t + i * 64];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) hraw[i] = sh[t + i * 64];
+  float val[NCH][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    unpack8(raw[i], val[i]);
+    float part = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) part += val[i][j];
+    sum += part;
+  }
+  const float mean = wave_sum(sum) / (float)(NCH * 512);
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    float part = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      val[i][j] -= mean;
+      part += val[i][j] * val[i][j];
+    }
+    sq += part;
+  }
+  const float rstd = rsqrtf(wave_sum(sq) / (float)(NCH * 512) + eps);
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    float s8[8], h8[8];
+    unpack8(sraw[i], s8);
+    unpack8(hraw[i], h8);
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      float v0 = val[i][j] * rstd, v1 = val[i][j + 1] * rstd;
+      round_bf16_pair_fused(v0, v1);
+      float a = 1.0f + s8[j], b = 1.0f + s8[j + 1];
+      round_bf16_pair_fused(a, b);
+      v0 *= a;
+      v1 *= b;
+      round_bf16_pair_fused(v0, v1);
+      v0 += h8[j];
+      v1 += h8[j + 1];
+      round_bf16_pair_fused(v0, v1);
+      val[i][j] = v0;
+      val[i][j + 1] = v1;
+      amax = max3_abs(amax, v0, v1);
+    }
+  }
+  amax = fmaxf(wave_max(amax), 1e-12f);
+  const float inv = 448.0f / amax;
+  if (t == 0) q_scale[row] = amax / 448.0f;
+  u32x2* qr = reinterpret_cast<u32x2*>(q + row * ldq);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) qr[t + i * 64] = quant8(val[i], inv);
 }
 
 // RMSNorm over the whole row followed by an optional per-head RoPE (head dim 128, pairs (2i, 2i+1)):
@@ -347,7 +424,11 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(const uint16_t* __restri
     unpack8(raw[i], val[i]);
     if (c >= npre) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) val[i][j] = round_bf16(ERF ? gelu_erf_f32(val[i][j]) : gelu_tanh_f32(val[i][j]));
+      for (int j = 0; j < 8; j += 2) {
+        val[i][j] = ERF ? gelu_erf_f32(val[i][j]) : gelu_tanh_f32(val[i][j]);
+        val[i][j + 1] = ERF ? gelu_erf_f32(val[i][j + 1]) : gelu_tanh_f32(val[i][j + 1]);
+        round_bf16_pair_fused(val[i][j], val[i][j + 1]);
+      }
     }
     if (c >= nchunk) {
 #pragma unroll
@@ -433,7 +514,11 @@ extern "C" int dsx_adaln_modulate(const void* x, int64_t ldx, const void* scale,
   // One wavefront per row while a row fits 6 chunks per lane and there are rows enough to fill the chip.
   // Wider rows: 12 chunks per lane cost 217 registers, two waves per SIMD and 266 us for 32760 x 5120; a
   // workgroup per row takes 160-175 us, a pair of wavefronts per row (two rows per workgroup) 145-150 us.
-  if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_ADALN(6, 64);
+  if (D == 512 * 6 && rows >= 1024 && scale && shift && !ln_w && !ln_b && q && q_scale && !y)
+    adaln_quant_rows_kernel<6><<<dim3((unsigned)((rows + 3) / 4)), block, 0, st>>>(
+        (const uint16_t*)x, ldx, (const uint16_t*)scale, (const uint16_t*)shift, mod_sb, rows_per_batch, eps,
+        (uint8_t*)q, ldq, q_scale, rows);
+  else if (D <= 512 * 6 && rows >= 1024) DSX_LAUNCH_ADALN(6, 64);
   else if (D <= 2048 * 2) DSX_LAUNCH_ADALN(2, 256);
   else if (D <= 1024 * 5 && rows >= 2048) DSX_LAUNCH_ADALN(5, 128);
   else if (D <= 2048 * 3) DSX_LAUNCH_ADALN(3, 256);
