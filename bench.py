@@ -187,10 +187,10 @@ def run_wan(torch, dev, layers, steps, warmup, with_cpu_baseline):
         "data": "synthetic",
         "config": {"workload": "BASELINE configs[4]: Wan2.1-14B-architecture DiT, one denoising step, %d layers, "
                                "32760 video tokens (21x60x104 latent) + 512 text tokens, batch 1, random init" % L},
-        # dominant kernel: attn_plain_kernel (53 % of the step's flops); self- and cross-attention launches together
+        # dominant kernel: attn_plain16_kernel (53 % of the step's flops); self- and cross-attention launches together
         "roofline": {"bound": "mfma", "achieved": round(attn_flops / attn_secs / 1e12, 1), "peak": PEAK_BF16 / 1e12,
                      "unit": "TFLOP/s", "frac": round(attn_flops / attn_secs / PEAK_BF16, 4),
-                     "traffic": WAN_ATTN_TRAFFIC_BYTES, "kernel": "attn_plain_kernel", "launches": n_attn,
+                     "traffic": WAN_ATTN_TRAFFIC_BYTES, "kernel": "attn_plain16_kernel", "launches": n_attn,
                      "avg_launch_us": round(attn_secs / max(n_attn, 1) * 1e6, 1)},
         "detail": {"fp8_gemm_in_step": {"launches": n_gemm, "tflops": round(gemm_flops / gemm_secs / 1e12, 1),
                                         "frac_fp8_peak": round(gemm_flops / gemm_secs / PEAK_FP8, 4),
@@ -581,15 +581,15 @@ def wan_cpu_baseline(cfg, S_full, S_sample=2048, reps=2):
 
 
 # L2-miss bytes per fp8_gemm_kernel launch, averaged over the 152 block-GEMM launches of one 19+38 step (the
-# image/text pairs of the joint blocks share a launch): rocprofv3 --pmc FETCH_SIZE (380.3 MB) plus --pmc WRITE_SIZE
+# image/text pairs of the joint blocks share a launch): rocprofv3 --pmc FETCH_SIZE (381.3 MB) plus --pmc WRITE_SIZE
 # (88.5 MB), each scaled by what the same counter reads for the 256 MiB copy of --calibrate-copy (FETCH_SIZE
 # counts half the copied bytes, WRITE_SIZE all of them); profiles/flux_step_hbm_traffic_pmc.txt holds the
 # per-shape figures.
-GEMM_TRAFFIC_BYTES = 468.8e6
+GEMM_TRAFFIC_BYTES = 469.8e6
 # L2-miss bytes per attention call of the Wan step, averaged over its self- and cross-attention calls (one of each
 # per layer): FETCH_SIZE + WRITE_SIZE runs of `--workload wan14b --wan-layers 2 --calibrate-copy`, scaled the same
-# way (profiles/wan14b_attention_hbm_traffic_pmc.txt: self-attention 3035 + 335 MB, cross-attention 363 + 336 MB).
-WAN_ATTN_TRAFFIC_BYTES = 2034.7e6
+# way (profiles/wan14b_attention_hbm_traffic_pmc.txt: self-attention 3025 + 335 MB, cross-attention 363 + 335 MB).
+WAN_ATTN_TRAFFIC_BYTES = 2029.0e6
 
 
 def main():
