@@ -456,6 +456,76 @@ def micro_benchmarks(torch, ops, dev):
     return detail
 
 
+def two_stream_overlap(torch, ops, dev, graph=True, pairs=20):
+    """Does a bandwidth-bound row kernel hide under an attention call?  In a single block GELU + quantise of the MLP
+    half and the attention call are independent (flux_dit.py:312-317).  Times, at the step's shapes: each kernel
+    alone, the pair back to back on one stream, and the pair with the row kernel forked onto a second stream of the
+    same priority (events for fork and join), as one recorded sequence of `pairs` pairs."""
+    g = torch.Generator(device=dev).manual_seed(0)
+    H, S = HEADS, N_IMG + N_TXT
+    q, k, v = [torch.randn(1, H, S, HEAD_DIM, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(3)]
+    q = torch.nn.functional.normalize(q.float(), dim=-1).mul(HEAD_DIM ** 0.5).bfloat16()
+    k = torch.nn.functional.normalize(k.float(), dim=-1).mul(HEAD_DIM ** 0.5).bfloat16()
+    out = torch.empty(1, S, H, HEAD_DIM, dtype=torch.bfloat16, device=dev).transpose(1, 2)
+    hs = [torch.randn(S, 4 * HIDDEN, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(4)]
+    side = torch.cuda.Stream()  # default priority
+
+    def attn():
+        ops.attention_bhsd(q, k, v, out=out, score_bound=1.02 * HEAD_DIM ** 0.5)
+
+    def gelu(i):
+        ops.gelu_tanh(hs[i % 4], want_bf16=False, want_fp8=True)
+
+    def only_attn(n):
+        for _ in range(n):
+            attn()
+
+    def only_gelu(n):
+        for i in range(n):
+            gelu(i)
+
+    def sequential(n):
+        for i in range(n):
+            attn()
+            gelu(i)
+
+    def forked(n):
+        main = torch.cuda.current_stream()
+        for i in range(n):
+            side.wait_stream(main)
+            attn()
+            with torch.cuda.stream(side):
+                gelu(i)
+            main.wait_stream(side)
+
+    def timeit(fn):
+        fn(3)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if graph:
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                fn(pairs)
+            gr.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(5):
+                gr.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / (5 * pairs)
+        e0.record()
+        fn(pairs)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / pairs
+
+    return {"attention_us": round(timeit(only_attn), 1), "gelu_quantise_us": round(timeit(only_gelu), 1),
+            "pair_on_one_stream_us": round(timeit(sequential), 1),
+            "pair_with_row_kernel_on_second_stream_us": round(timeit(forked), 1),
+            "timed_as": "graph replay" if graph else "eager launches"}
+
+
 def cpu_baseline(num_double, num_single):
     """The oracle (fp32, torch SDPA-equivalent eager attention) on the host cores: ONE double-stream and ONE
     single-stream block at the full 4096+512 tokens, extrapolated to 19 + 38 blocks."""
@@ -604,6 +674,9 @@ def main():
     ap.add_argument("--workload", choices=("flux", "wan14b"), default="flux",
                     help="flux (default): the headline Flux-1024 step; wan14b: one Wan2.1-14B step (configs[4])")
     ap.add_argument("--wan-layers", type=int, default=40)
+    ap.add_argument("--overlap-probe", action="store_true",
+                    help="only run the two-stream overlap probe (attention beside GELU + quantise) with eager "
+                         "launches, for a kernel trace of it, and print its figures")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy, the known-size dispatch that FETCH_SIZE / "
                          "WRITE_SIZE counter runs are scaled by")
@@ -629,6 +702,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.overlap_probe:
+        print(json.dumps({"two_stream_overlap": two_stream_overlap(torch, ops, dev, graph=False)}))
+        return
     if args.workload == "wan14b":
         print(json.dumps(run_wan(torch, dev, args.wan_layers, args.steps, args.warmup, not args.no_cpu_baseline)))
         return
@@ -697,6 +773,7 @@ def main():
         "fp8_gemm_in_step": {"ms_per_step": round(gemm_secs * 1e3 / args.steps, 2)}}
     if not args.no_micro:
         result["detail"].update(micro_benchmarks(torch, ops, dev))
+        result["detail"]["two_stream_overlap"] = two_stream_overlap(torch, ops, dev)
         probe = mfma_ceiling(torch, dev)
         result["detail"]["mfma_ceiling_probe"] = probe
         # The same step against what THIS box's matrix pipes sustain on random operand bits (bare MFMA streams, every
