@@ -139,10 +139,15 @@ def run_wan(torch, dev, layers, steps, warmup, with_cpu_baseline):
     t = torch.tensor([500.0], device=dev)
     from diffsynth_engine_amd import ops
 
-    for _ in range(args.warmup):
-        out = runner(x, ctx, t)
+    at, gt = AttnTimer(torch, ops), GemmTimer(torch, ops)
+    with at, gt:  # bracketed like the timed steps: says how many events a step takes, and creates the first of them
+        for _ in range(args.warmup):
+            out = runner(x, ctx, t)
+    if args.warmup:
+        at.prepare(len(at.records) // args.warmup * args.steps)
+        gt.prepare(len(gt.records) // args.warmup * args.steps)
     torch.cuda.synchronize()
-    with AttnTimer(torch, ops) as at, GemmTimer(torch, ops) as gt:
+    with at, gt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             out = runner(x, ctx, t)
@@ -212,40 +217,71 @@ def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
     return gemm, attn
 
 
-class GemmTimer:
-    """Brackets every fp8_gemm launch (single, or two problems sharing one grid) with events on the launch
-    stream (torch's current stream, which is the stream handed to the C-ABI) and accumulates algorithmic
-    flops for launches with M > 8."""
+class _EventBrackets:
+    """Event pairs around calls on the launch stream (torch's current stream, which is the stream handed to the
+    C-ABI), with the flops of each call.
+
+    Events come from a pool that `prepare` fills BEFORE a timed region: the first record of a new timing event
+    makes the HIP runtime allocate its signal, hundreds at a time cost the host tens of milliseconds (30 ms in one
+    piece in the first GPU process of a freshly started machine), and a timed region of five steps that creates its
+    3100 events as it goes is host-bound through its first step and reads 3-6 ms per step more than the steps take."""
 
     def __init__(self, torch, ops):
         self.torch, self.ops = torch, ops
-        self.records = []
+        self.records, self.pool = [], []
+
+    def _pair(self):
+        if self.pool:
+            return self.pool.pop()
+        return self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+
+    def prepare(self, pairs):
+        """Leaves `pairs` event pairs in the pool, each recorded once (that is what creates them), keeps the pairs
+        of earlier records for re-use and forgets those records."""
+        self.pool += [(e0, e1) for e0, e1, _ in self.records]
+        del self.records[:]
+        while len(self.pool) < pairs:
+            e0, e1 = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+            e0.record()
+            e1.record()
+            self.pool.append((e0, e1))
+        self.torch.cuda.synchronize()
+
+    def bracket(self, fn, flops):
+        e0, e1 = self._pair()
+        e0.record()
+        out = fn()
+        e1.record()
+        self.records.append((e0, e1, flops))
+        return out
+
+    def summary(self):
+        self.torch.cuda.synchronize()
+        secs = sum(e0.elapsed_time(e1) for e0, e1, _ in self.records) * 1e-3
+        return len(self.records), sum(f for _, _, f in self.records), secs
+
+
+class GemmTimer(_EventBrackets):
+    """Brackets every fp8_gemm launch (single, or two problems sharing one grid) and accumulates algorithmic flops
+    for launches with M > 8."""
+
+    def __init__(self, torch, ops):
+        super().__init__(torch, ops)
         self._orig = ops.fp8_gemm
         self._orig_grouped = ops.fp8_gemm_grouped
 
     def __enter__(self):
-        torch, orig, rec = self.torch, self._orig, self.records
+        orig, orig_grouped = self._orig, self._orig_grouped
 
         def timed(a_q, w_q, *args, **kw):
             M, K = a_q.shape
             if M <= 8 or kw.get("qk") is not None:  # (a q/k-epilogue call goes through the grouped entry, timed there)
                 return orig(a_q, w_q, *args, **kw)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            out = orig(a_q, w_q, *args, **kw)
-            e1.record()
-            rec.append((e0, e1, 2.0 * M * K * w_q.shape[0]))
-            return out
-
-        orig_grouped = self._orig_grouped
+            return self.bracket(lambda: orig(a_q, w_q, *args, **kw), 2.0 * M * K * w_q.shape[0])
 
         def timed_grouped(problems):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            out = orig_grouped(problems)
-            e1.record()
-            rec.append((e0, e1, sum(2.0 * p["a_q"].shape[0] * p["a_q"].shape[1] * p["w_q"].shape[0] for p in problems)))
-            return out
+            return self.bracket(lambda: orig_grouped(problems),
+                                sum(2.0 * p["a_q"].shape[0] * p["a_q"].shape[1] * p["w_q"].shape[0] for p in problems))
 
         self.ops.fp8_gemm = timed
         self.ops.fp8_gemm_grouped = timed_grouped
@@ -255,45 +291,29 @@ class GemmTimer:
         self.ops.fp8_gemm = self._orig
         self.ops.fp8_gemm_grouped = self._orig_grouped
 
-    def summary(self):
-        self.torch.cuda.synchronize()
-        secs = sum(e0.elapsed_time(e1) for e0, e1, _ in self.records) * 1e-3
-        flops = sum(f for _, _, f in self.records)
-        return len(self.records), flops, secs
 
-
-class AttnTimer:
-    """Brackets every ops.attention_bhsd call of a step with events on the launch stream and accumulates the
-    algorithmic flops 4 * Sq * Skv * D * H * B of each (a call with fused q/k pre-processing includes its k row pass)."""
+class AttnTimer(_EventBrackets):
+    """Brackets every ops.attention_bhsd call of a step and accumulates the algorithmic flops
+    4 * Sq * Skv * D * H * B of each (a call with fused q/k pre-processing includes its k row pass)."""
 
     def __init__(self, torch, ops):
-        self.torch, self.ops, self.records = torch, ops, []
+        super().__init__(torch, ops)
         self._orig = ops.attention_bhsd
 
     def __enter__(self):
-        torch, orig, rec = self.torch, self._orig, self.records
+        orig = self._orig
 
         def timed(q, k, v, *args, q2=None, k2=None, **kw):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            out = orig(q, k, v, *args, q2=q2, k2=k2, **kw)
-            e1.record()
             B, H, Sq, D = q.shape
             Sq += 0 if q2 is None else q2.shape[2]
             Skv = k.shape[2] + (0 if k2 is None else k2.shape[2])
-            rec.append((e0, e1, 4.0 * B * H * Sq * Skv * D))
-            return out
+            return self.bracket(lambda: orig(q, k, v, *args, q2=q2, k2=k2, **kw), 4.0 * B * H * Sq * Skv * D)
 
         self.ops.attention_bhsd = timed
         return self
 
     def __exit__(self, *exc):
         self.ops.attention_bhsd = self._orig
-
-    def summary(self):
-        self.torch.cuda.synchronize()
-        secs = sum(e0.elapsed_time(e1) for e0, e1, _ in self.records) * 1e-3
-        return len(self.records), sum(f for _, _, f in self.records), secs
 
 
 def time_kernel(torch, fn, args_list=None, reps=10):
@@ -720,10 +740,14 @@ def main():
         guidance=torch.tensor([3.5], device=dev),
         text_ids=torch.zeros(1, N_TXT, 3, device=dev),
     )
-    for _ in range(args.warmup):
-        out = runner(**inp)
+    gt = GemmTimer(torch, ops)
+    with gt:  # bracketed like the timed steps: says how many events a step takes, and creates the first of them
+        for _ in range(args.warmup):
+            out = runner(**inp)
+    if args.warmup:
+        gt.prepare(len(gt.records) // args.warmup * args.steps)
     torch.cuda.synchronize()
-    with GemmTimer(torch, ops) as gt:
+    with gt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             out = runner(**inp)
