@@ -60,9 +60,9 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
         if constexpr (KIND == 0)
           acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
                                                            acc[t], 0, 0, 0);
-        else
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
-                                                           acc[t], 0, 0, 0);
+        else  // as assembly with the accumulator tied to itself: for this shape the compiler's own allocation puts
+              // source and destination accumulators in different registers and copies them around once per round
+          asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[t]) : "v"(a), "v"(b));
       } else {
         const i32x8 a = {(int)r[ra], (int)r[ra + 1], (int)r[ra + 2], (int)r[ra + 3], (int)r[ra + 4], (int)r[ra + 5],
                          (int)r[ra + 6], (int)r[ra + 7]};
@@ -75,6 +75,7 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(const uint32_t* __res
       }
     }
   }
+  if constexpr (KIND == 2) asm volatile("s_nop 15\n\ts_nop 15");  // (the assembly MFMAs' results, before they are read)
   float s = 0.f;
 #pragma unroll
   for (int t = 0; t < kAcc; ++t)
