@@ -424,7 +424,8 @@ def micro_benchmarks(torch, ops, dev):
     out = torch.empty(1, S, HEADS, HEAD_DIM, dtype=torch.bfloat16, device=dev).transpose(1, 2)
     fl = 4.0 * S * S * HEAD_DIM * HEADS
     t = time_kernel(torch, lambda: ops.attention_bhsd(q, k, v, out=out))
-    att = {"plain": {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1), "frac_bf16_peak": round(fl / t / PEAK_BF16, 4)}}
+    att = {"plain": {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1), "frac_bf16_peak": round(fl / t / PEAK_BF16, 4),
+                     "kernel_launches": 1}}
     # fused RMSNorm + 3-axis RoPE (16,56,56), ids: 512 text rows at 0, then (0,r,c) over 64x64
     ids = torch.zeros(1, S, 3, dtype=torch.float64, device=dev)
     rc = torch.arange(64, device=dev, dtype=torch.float64)
@@ -446,7 +447,8 @@ def micro_benchmarks(torch, ops, dev):
         t = time_kernel(torch, lambda: ops.attention_bhsd(q, k, v, out=out, rope=rope, q_norm_w=w1, k_norm_w=w1,
                                                           score_bound=bound))
         att[key] = {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
-                    "frac_bf16_peak": round(fl / t / PEAK_BF16, 4)}
+                    "frac_bf16_peak": round(fl / t / PEAK_BF16, 4),
+                    "kernel_launches": 2}  # one C call, two launches: the k row pass, then attention (q as it loads)
     detail["attention_S4608_H24_D128"] = att
 
     mod = torch.randn(1, 3 * HIDDEN, generator=g, device=dev, dtype=torch.bfloat16)
