@@ -673,11 +673,11 @@ def wan_cpu_baseline(cfg, S_full, S_sample=2048, reps=2):
 
 
 # L2-miss bytes per fp8_gemm_kernel launch, averaged over the 152 block-GEMM launches of one 19+38 step (the
-# image/text pairs of the joint blocks share a launch): rocprofv3 --pmc FETCH_SIZE (381.3 MB) plus --pmc WRITE_SIZE
+# image/text pairs of the joint blocks share a launch): rocprofv3 --pmc FETCH_SIZE (383.0 MB) plus --pmc WRITE_SIZE
 # (88.5 MB), each scaled by what the same counter reads for the 256 MiB copy of --calibrate-copy (FETCH_SIZE
 # counts half the copied bytes, WRITE_SIZE all of them); profiles/flux_step_hbm_traffic_pmc.txt holds the
 # per-shape figures.
-GEMM_TRAFFIC_BYTES = 469.8e6
+GEMM_TRAFFIC_BYTES = 471.5e6
 # L2-miss bytes per attention call of the Wan step, averaged over its self- and cross-attention calls (one of each
 # per layer): FETCH_SIZE + WRITE_SIZE runs of `--workload wan14b --wan-layers 2 --calibrate-copy`, scaled the same
 # way (profiles/wan14b_attention_hbm_traffic_pmc.txt: self-attention 3025 + 335 MB, cross-attention 363 + 335 MB).
