@@ -217,6 +217,51 @@ def step_flops(num_double, num_single, n_img=N_IMG, n_txt=N_TXT):
     return gemm, attn
 
 
+_HIP = None
+
+
+def _hip_runtime():
+    """The HIP runtime this process already has loaded (torch's), through ctypes: for timing events with flags that
+    torch.cuda.Event does not expose."""
+    global _HIP
+    if _HIP is None:
+        import ctypes
+
+        path = next(tok for tok in open("/proc/self/maps").read().split() if "libamdhip64" in tok)
+        hip = ctypes.CDLL(path)
+        hip.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+        hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        _HIP = hip
+    return _HIP
+
+
+class _HipEvent:
+    """A HIP timing event without the system-scope fence of a default event (hipEventDisableSystemFence): the
+    brackets around the 155 GEMM launches of a step then cost 0.45 ms per step instead of 1.0 ms, and a bracket
+    holds 2 us less that is not the kernel."""
+
+    def __init__(self, torch):
+        import ctypes
+
+        self._ct, self._torch, self.h = ctypes, torch, ctypes.c_void_p()
+        rc = _hip_runtime().hipEventCreateWithFlags(ctypes.byref(self.h), 0x20000000)  # hipEventDisableSystemFence
+        if rc:
+            raise RuntimeError("hipEventCreateWithFlags failed: %d" % rc)
+
+    def record(self):  # on torch's current stream, the stream handed to the C-ABI
+        rc = _hip_runtime().hipEventRecord(self.h, self._ct.c_void_p(self._torch.cuda.current_stream().cuda_stream))
+        if rc:
+            raise RuntimeError("hipEventRecord failed: %d" % rc)
+
+    def elapsed_time(self, later):  # ms
+        ms = self._ct.c_float()
+        rc = _hip_runtime().hipEventElapsedTime(self._ct.byref(ms), self.h, later.h)
+        if rc:
+            raise RuntimeError("hipEventElapsedTime failed: %d" % rc)
+        return ms.value
+
+
 class _EventBrackets:
     """Event pairs around calls on the launch stream (torch's current stream, which is the stream handed to the
     C-ABI), with the flops of each call.
@@ -230,10 +275,11 @@ class _EventBrackets:
         self.torch, self.ops = torch, ops
         self.records, self.pool = [], []
 
+    def _new_pair(self):
+        return _HipEvent(self.torch), _HipEvent(self.torch)
+
     def _pair(self):
-        if self.pool:
-            return self.pool.pop()
-        return self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+        return self.pool.pop() if self.pool else self._new_pair()
 
     def prepare(self, pairs):
         """Leaves `pairs` event pairs in the pool, each recorded once (that is what creates them), keeps the pairs
@@ -241,7 +287,7 @@ class _EventBrackets:
         self.pool += [(e0, e1) for e0, e1, _ in self.records]
         del self.records[:]
         while len(self.pool) < pairs:
-            e0, e1 = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+            e0, e1 = self._new_pair()
             e0.record()
             e1.record()
             self.pool.append((e0, e1))
