@@ -899,27 +899,52 @@ def main():
         # the same step with an unfused rank-16 LoRA on every one of the 228 block linears (LoRALinear.forward,
         # models/basic/lora.py:137-141): the updates ride the main products as 128 more columns of their reduction
         # axis, one small down-projection launch per linear
+        def plain_steps(n=5):  # ms per step without event brackets (the headline's timed region carries them)
+            for _ in range(2):
+                runner(**inp)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                o = runner(**inp)
+            torch.cuda.synchronize()
+            assert torch.isfinite(o.float()).all().item(), "non-finite output"
+            return (time.perf_counter() - t0) * 1e3 / n
+
+        ms_plain = plain_steps()
         names = [n for n in runner.lin if n.startswith(("blocks.", "single_blocks."))]
         for n in names:
             L = runner.lin[n]
             L.add_lora((torch.randn(16, L.k, generator=g, device=dev) * 0.01).to(torch.bfloat16),
                        (torch.randn(L.n, 16, generator=g, device=dev) * 0.01).to(torch.bfloat16), 1.0)
         riding = sum(runner.lin[n]._extension() is not None for n in names)
-        for _ in range(2):
-            out_l = runner(**inp)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(5):
-            out_l = runner(**inp)
-        torch.cuda.synchronize()
-        ms_l = (time.perf_counter() - t0) * 1e3 / 5
-        assert torch.isfinite(out_l.float()).all().item(), "non-finite output"
+        ms_l = plain_steps()
         result["detail"]["lora_rank16_on_all_block_linears"] = {
             "linears": len(names), "riding_the_main_product": riding, "ms_per_step": round(ms_l, 2),
-            "overhead_frac": round(ms_l / ms - 1.0, 4)}
+            "ms_per_step_without_lora_same_timing": round(ms_plain, 2),
+            "overhead_frac": round(ms_l / ms_plain - 1.0, 4)}
     del runner
     torch.cuda.empty_cache()
     if not args.no_micro:
+        # the same step in the reference's own fp8 arithmetic (utils/fp8_linear.py:28-60: bare e4m3 casts, unit
+        # scales), weights drawn N(0, 1/fan_in) so that no activation comes near e4m3's 448, next to the scaled
+        # mode on the same weights: what the per-token scales of the headline mode cost
+        unit = {}
+        for mode, scaled in (("unit_scales", False), ("per_token_scales", True)):
+            r2 = FluxDiTRunner(flux_state_dict_stream(args.double, args.single, dev, std=None), args.double,
+                               args.single, scaled=scaled, device=dev)
+            for _ in range(2):
+                out_u = r2(**inp)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                out_u = r2(**inp)
+            torch.cuda.synchronize()
+            unit[mode + "_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / 5, 2)
+            assert torch.isfinite(out_u.float()).all().item(), "non-finite output"
+            del r2
+            torch.cuda.empty_cache()
+        unit["weights"] = "N(0, 1/fan_in), AdaLN projections at half that deviation"
+        result["detail"]["flux_step_in_the_references_arithmetic"] = unit
         # BASELINE configs[4] beside the headline figure: the whole Wan2.1-14B step, all 40 layers at 32 760 + 512
         # tokens, same code path as `--workload wan14b` (one warm-up step, two timed ones; a step is about a second)
         w = run_wan(torch, dev, 40, 2, 1, not args.no_cpu_baseline)
