@@ -423,3 +423,30 @@ def test_lora_down_against_the_fp32_product(dev, M, K, R):
     step = wf.abs().clamp_min(2 ** -6) * 0.125
     assert ((gf - ref.clamp(-448, 448)).abs() <= step)[:, : R - 1].all()
     assert (got[:, copies * R:].view(torch.uint8) == 0).all()
+
+
+@pytest.mark.parametrize("ranks", [4, 16, 20, 48, 80, 112])
+def test_lora_down_every_rank_tile_count(dev, ranks):
+    """Every number of 16-rank tiles (1 to 8) has its own instantiation with its own buffer depth and wavefront count;
+    ragged row counts (not a multiple of the 16-row tile) and K of one to many chunks per wavefront."""
+    from diffsynth_engine_amd import ops
+
+    R = (ranks + 31) // 32 * 32
+    for M, K in ((70, 128), (33, 640), (257, 3072)):
+        g = torch.Generator().manual_seed(ranks * 1000 + M + K)
+        a = torch.randn(M, K, generator=g).mul(60).to(dev).to(ops.FP8)
+        d = torch.zeros(R, K)
+        d[:ranks] = torch.randn(ranks, K, generator=g).mul(60)
+        d = d.to(dev).to(ops.FP8)
+        rs = (torch.rand(R, generator=g) + 0.5).mul(100.0 / (60 * 60 * K ** 0.5)).to(dev)
+        got = ops.lora_down(a, d, rs, 128, 1, ranks=ranks)
+        ref = ((a.double() @ d.double().t()) * rs.double()).float()[:, :ranks]
+        gf, wf = got[:, :ranks].float(), ref.clamp(-448, 448).to(ops.FP8).float()
+        assert torch.isfinite(gf).all()
+        assert (gf != wf).float().mean().item() < 5e-3, (M, K)
+        # one grid step, or -- for values near zero, whose steps are tiny -- the matrix pipe's accumulation error:
+        # about 1e-5 of the magnitude that went through the sum
+        mag = ((a.float().abs() @ d.float().abs().t()) * rs)[:, :ranks]
+        tol = torch.maximum(wf.abs().clamp_min(2 ** -6) * 0.125, 1e-5 * mag)
+        assert ((gf - ref.clamp(-448, 448)).abs() <= tol).all(), (M, K)
+        assert (got[:, ranks:].view(torch.uint8) == 0).all()
