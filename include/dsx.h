@@ -160,7 +160,8 @@ int dsx_fp8_gemm_grouped(const dsx_gemm_problem* problems, int count, void* stre
  * columns of w_ext (1 / copies included: writing a row's values `copies` times, against as many repeats of w_ext's
  * columns, keeps each of them that much further from e4m3's end).
  * R % 32 == 0, R <= 128, ranks % 4 == 0, ranks <= R, 1 <= copies <= 32, E >= copies * ranks, E % 16 == 0,
- * K % 128 == 0.
+ * K % 128 == 0, lda and ldd below 2^24 (DSX_EBADSHAPE otherwise); a, d, out and their leading dimensions 16-byte
+ * aligned (DSX_EALIGN).
  * Replaces `lora.down(x)` of LoRA.forward (diffsynth_engine/models/basic/lora.py:29-32) for every update of a layer
  * in one HBM-bound pass over a.
  */
