@@ -275,8 +275,15 @@ class _EventBrackets:
         self.torch, self.ops = torch, ops
         self.records, self.pool = [], []
 
+    kind = "hip events without system-scope fence"
+
     def _new_pair(self):
-        return _HipEvent(self.torch), _HipEvent(self.torch)
+        if _EventBrackets.kind.startswith("hip"):
+            try:
+                return _HipEvent(self.torch), _HipEvent(self.torch)
+            except (StopIteration, OSError, AttributeError, RuntimeError):  # runtime not found through /proc: torch's
+                _EventBrackets.kind = "torch.cuda.Event"
+        return self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
 
     def _pair(self):
         return self.pool.pop() if self.pool else self._new_pair()
@@ -833,7 +840,7 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP8, 4),
                      "traffic": GEMM_TRAFFIC_BYTES if (args.double, args.single) == (19, 38) else None,
                      "kernel": "fp8_gemm_kernel", "launches": n_gemm,
-                     "avg_launch_us": round(gemm_secs / max(n_gemm, 1) * 1e6, 1)},
+                     "avg_launch_us": round(gemm_secs / max(n_gemm, 1) * 1e6, 1), "timed_with": _EventBrackets.kind},
         "step_roofline": {"algorithmic_tflop": round((gemm_fl + attn_fl) / 1e12, 2),
                           "ideal_ms": round(t_ideal * 1e3, 2), "frac": round(t_ideal * 1e3 / ms, 4)},
     }
