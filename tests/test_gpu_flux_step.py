@@ -369,3 +369,35 @@ def test_lora_forms_are_equally_close_to_the_exact_update(dev, M, K, N, r, std, 
     strong = _Linear(W, None, True)
     strong.add_lora(D * 64, U, coef)
     assert strong._extension() is None
+
+
+def test_rope_table_is_kept_only_while_the_ids_are_untouched(dev):
+    """The runner keeps the RoPE table of its last call while the id tensors are the same unmodified objects (a
+    denoising loop); an in-place change of the ids, other id tensors or another latent size rebuild it."""
+    from diffsynth_engine_amd.flux_dit import FluxDiTRunner
+
+    sd = oflux.init_params(1, 1, dtype=torch.bfloat16, seed=41, bias_std=0.02)
+    runner = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)
+    fresh = FluxDiTRunner(sd, 1, 1, scaled=True, device=dev)  # never sees the same id objects twice
+    inp = {k: v.to(dev) for k, v in _inputs(16, 24, seed=42).items()}
+
+    def once(r, **kw):
+        return r(**dict(inp, **kw))
+
+    first = once(runner)
+    table = runner._rope_table
+    assert torch.equal(once(runner), first) and runner._rope_table is table  # second step: the table is reused
+    inp["text_ids"][0, :, 1] += 3.0  # the same tensor object, modified in place
+    moved = once(runner)
+    assert runner._rope_table is not table
+    assert torch.equal(moved, once(fresh, text_ids=inp["text_ids"].clone()))
+    assert not torch.equal(moved, first)
+    ids = torch.zeros(1, 64, 3, device=dev)
+    ids[0, :, 1] = torch.arange(64, device=dev) // 8 + 5  # explicit image ids, shifted rows
+    ids[0, :, 2] = torch.arange(64, device=dev) % 8
+    shifted = once(runner, image_ids=ids)
+    assert torch.equal(shifted, once(fresh, image_ids=ids.clone()))
+    assert not torch.equal(shifted, moved)
+    # another latent size with the same text ids
+    other = dict(inp, hidden_states=torch.randn(1, 16, 16, 32, device=dev).bfloat16())
+    assert torch.equal(runner(**other), fresh(**dict(other, text_ids=inp["text_ids"].clone())))
