@@ -93,3 +93,28 @@ def test_row_kernels_refuse_operands_that_do_not_fit(dev):
     with pytest.raises(ValueError):
         ops.gated_residual(rows, rows, torch.ones(3, 256, device=dev, dtype=BF))
     assert torch.equal(ops.gated_residual(rows, torch.zeros_like(rows), torch.ones(1, 256, device=dev)), rows)
+
+
+def test_lora_down_refuses_operands_that_do_not_fit(dev):
+    """ops.lora_down on the host, dsx_lora_down in the library: sizes the kernel's tiles and its 16-byte loads do not
+    cover come back as an error before anything is launched."""
+    from diffsynth_engine_amd import ops
+
+    a = torch.randn(48, 256, device=dev).mul(50).to(F8)
+    d = torch.randn(32, 256, device=dev).mul(50).to(F8)
+    rs = torch.full((32,), 1e-4, device=dev)
+    assert ops.lora_down(a, d, rs, 128, 4).shape == (48, 128)
+    bad = [dict(d_q=d[:, :128]),                                   # K of the factors differs
+           dict(a_q=a.to(BF)),                                     # not e4m3
+           dict(row_scale=rs[:16]), dict(row_scale=rs.double()),   # one fp32 scale per row of d
+           dict(d_q=d[:16].contiguous(), row_scale=rs[:16].contiguous()),  # rows of d: a multiple of 32
+           dict(copies=5),                                         # 5 x 32 columns do not fit 128
+           dict(copies=0), dict(ranks=6), dict(ranks=40),          # ranks: a multiple of 4, at most the rows of d
+           dict(a_q=a[:, :192], d_q=d[:, :192].contiguous()),      # K: a multiple of 128
+           dict(width=120)]                                        # output width: a multiple of 16
+    for kw in bad:
+        args = dict(a_q=a, d_q=d, row_scale=rs, width=128, copies=4)
+        args.update(kw)
+        with pytest.raises((ValueError, RuntimeError)):
+            ops.lora_down(**args)
+    assert ops.lora_down(a[:0], d, rs, 128, 4).shape == (0, 128)  # no rows: nothing to do
