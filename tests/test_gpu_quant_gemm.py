@@ -370,6 +370,32 @@ def test_k_extension_equals_the_concatenated_operands(dev, kind, M):
     assert not torch.equal(ops.fp8_gemm(a1, w1, xs, ws, bias, **kw), whole)
 
 
+def test_a_pair_with_one_extended_problem_shares_a_launch(dev):
+    """Two problems in one grid (the image and text linears of a joint block) of which only one continues its
+    reduction axis, in either position, with different K: each gets the bits of its own single launch."""
+    from diffsynth_engine_amd import ops
+
+    g = torch.Generator().manual_seed(5)
+
+    def problem(M, K, N, ext):
+        x = torch.randn(M, K, generator=g).bfloat16().to(dev)
+        w = (torch.randn(N, K, generator=g) * 0.05).bfloat16().to(dev)
+        wq, ws = ops.quantize_weight_fp8(w)
+        xq, xs = ops.quantize_fp8(x)
+        p = dict(a_q=xq, w_q=wq, a_scale=xs, w_scale=ws, bias=torch.randn(N, generator=g).bfloat16().to(dev))
+        if ext:
+            p["ext"] = (torch.randn(M, 128, generator=g).mul(40).to(dev).to(ops.FP8),
+                        torch.randn(N, 128, generator=g).mul(40).to(dev).to(ops.FP8))
+        return p
+
+    for first_ext in (True, False):
+        big, small = problem(1024, 768, 1024, first_ext), problem(200, 1280, 512, not first_ext)
+        together = ops.fp8_gemm_grouped([big, small])
+        for got, p in zip(together, (big, small)):
+            assert torch.equal(got, ops.fp8_gemm(p["a_q"], p["w_q"], p["a_scale"], p["w_scale"], p["bias"],
+                                                 ext=p.get("ext")))
+
+
 def test_k_extension_refusals(dev):
     from diffsynth_engine_amd import ops
 
